@@ -1,0 +1,136 @@
+/*
+ * C ABI of the MI355X planning library (liblplb_hip.so).
+ *
+ * Each entry point replaces one method of the reference's pybind11 class
+ * `lplb._cpp.CompiledSolver` (csrc/plugin.cpp:663-679 of the reference) and
+ * takes what that method's host code hands to its kernel: raw device pointers,
+ * sizes and the stream.  All pointers are device pointers on the current HIP
+ * device unless stated otherwise.  Inputs are borrowed, outputs are caller
+ * allocated; the library owns no user-visible memory.  Calls only enqueue work
+ * on `stream` (a hipStream_t passed as void*, NULL = the default stream) and
+ * never synchronise.
+ *
+ * Every function returns 0 on success or an LPLB_E* code; the message of the
+ * calling thread's last failure is available from lplb_last_error().  No C++
+ * exception crosses this boundary.  An LP that fails the feasibility test is
+ * not an error: its group gets the neutral split 0.5 and the feasible-solution
+ * counter is left unchanged, as in the reference (minilp.cu:379-400).
+ */
+#ifndef LPLB_HIP_H
+#define LPLB_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LPLB_ABI_VERSION 1
+
+#define LPLB_OK 0
+#define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
+#define LPLB_EUNSUPPORTED 2 /* shape outside what the kernels are built for */
+#define LPLB_EHIP 3        /* a HIP runtime call failed */
+
+/* Step-length rules of the affine-scaling iteration. */
+#define LPLB_STEP_REFERENCE_WINDOW 0 /* max over the last 32 columns, as minilp.cu:355-359 does */
+#define LPLB_STEP_FULL_MAX 1         /* max over all columns (and 0) */
+
+typedef void *lplb_stream_t;
+
+int lplb_abi_version(void);
+
+/* Message of this thread's most recent failing call ("" if none). Host pointer. */
+const char *lplb_last_error(void);
+
+/*
+ * Per-expert token histogram with an inclusive prefix over slices.
+ * Replaces CompiledSolver.count_idx (csrc/plugin.cpp:580-600, kernel
+ * minilp.cu:410-443).
+ *
+ *   idx              int64 [n_elements], values in [-1, n_experts); -1 (and any
+ *                    other out-of-range value) is not counted
+ *   n_blocks         number of slices (the reference's n_sms).  Slice p covers
+ *                    [min(n, per*p), min(n, per*(p+1))) with
+ *                    per = roundup(ceil(n / n_blocks), 256)  (minilp.cu:404-408)
+ *   counts_by_block  int32 [n_blocks, n_experts], out: row p = occurrences in
+ *                    slices 0..p.  The last row is the full histogram.
+ */
+int lplb_count_idx(const int64_t *idx, int64_t n_elements, int n_experts,
+                   int n_blocks, int32_t *counts_by_block, lplb_stream_t stream);
+
+/*
+ * Builds and solves one LP per EP group: minimise the maximum per-rank load by
+ * moving tokens along replica edges.  Replaces CompiledSolver.solve
+ * (csrc/plugin.cpp:491-578, kernel minilp.cu:83-402 without its NVSHMEM branch).
+ *
+ *   workload         int32 [n_group, group_size, L], global per-expert counts,
+ *                    L = dup_per_rank * n_experts_per_var + n_experts_fixed
+ *   global_workload  fp32 [n_group, group_size, L], out: counts / max count
+ *   r2o              int32 [group_size, dup_per_rank] replica topology
+ *   phy2log          int32 [n_group * group_size * P], P = L + dup_per_rank *
+ *                    n_experts_per_var; per rank: replicated originals (slot =
+ *                    c * dup_per_rank + d), other originals, replicas
+ *   avail_num        int32 [1], in/out: incremented once per group whose LP
+ *                    passed the feasibility test (never reset here)
+ *   result           fp32 [n_group, group_size, dup_per_rank], out: share of
+ *                    each replicated expert set that stays on its original rank
+ *   step_rule        LPLB_STEP_*; 0 reproduces the reference
+ *   n_steps          number of affine-scaling steps; the reference uses 5
+ *
+ * Requires group_size * dup_per_rank <= 64 (LPLB_EUNSUPPORTED otherwise).
+ */
+int lplb_solve(const int32_t *workload, float *global_workload,
+               const int32_t *r2o, const int32_t *phy2log, int n_group,
+               int group_size, int dup_per_rank, int n_experts_per_var,
+               int n_experts_fixed, int32_t *avail_num, float *result,
+               int step_rule, int n_steps, lplb_stream_t stream);
+
+/*
+ * n_instances independent lplb_solve problems that share r2o and phy2log, one
+ * wavefront per (instance, group), in a single launch.  No counterpart in the
+ * reference (it solves one batch per launch); workloads / global_workloads /
+ * results carry a leading [n_instances] dimension.  global_workloads may be
+ * NULL.  avail_num is incremented once per feasible (instance, group).
+ */
+int lplb_solve_batched(const int32_t *workloads, float *global_workloads,
+                       const int32_t *r2o, const int32_t *phy2log,
+                       int n_instances, int n_group, int group_size,
+                       int dup_per_rank, int n_experts_per_var,
+                       int n_experts_fixed, int32_t *avail_num, float *results,
+                       int step_rule, int n_steps, lplb_stream_t stream);
+
+/*
+ * Logical -> physical redirect of routing indices.  Replaces
+ * CompiledSolver.map_idx (csrc/plugin.cpp:602-660, kernel minilp.cu:445-515).
+ *
+ *   idx              int64 [n_elements] logical expert ids, -1 = masked
+ *   o_weight         fp32 [n_group, group_size, dup_per_rank] from lplb_solve
+ *   counts_by_block  int32 [n_blocks, n_logical] from lplb_count_idx on the
+ *                    same idx and n_blocks
+ *   o2r              int32 [group_size, dup_per_rank], column-wise inverse of r2o
+ *   phy2log          as for lplb_solve
+ *   n_combined_experts  replicated expert sets per replica slot (C)
+ *   n_local_experts  physical experts per rank (P)
+ *   out              int64 [n_elements]: -1 stays -1; token number k (counting
+ *                    earlier occurrences of the same expert in index order) of
+ *                    expert e goes to e's original slot if
+ *                    (499 k + 41) mod total[e] < trunc(o_weight * total[e]),
+ *                    else to its replica (minilp.cu:484-486, 503-509)
+ *
+ * The reference takes each token's k from a shared-memory atomic, so which
+ * token of a block gets which k is unspecified there; here k always follows
+ * index order, which makes the output deterministic and independent of
+ * n_blocks.  Values outside [-1, n_logical) map to -1.
+ */
+int lplb_map_idx(const int64_t *idx, const float *o_weight,
+                 const int32_t *counts_by_block, const int32_t *o2r,
+                 const int32_t *phy2log, int64_t n_elements, int n_group,
+                 int group_size, int dup_per_rank, int n_combined_experts,
+                 int n_local_experts, int n_blocks, int64_t *out,
+                 lplb_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LPLB_HIP_H */

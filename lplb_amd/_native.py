@@ -1,0 +1,204 @@
+"""ctypes binding of ``liblplb_hip.so`` and the ``CompiledSolver`` facade the planner
+talks to.  The facade keeps the method names, argument order, return values and
+argument checks of the reference's pybind11 class (csrc/plugin.cpp:459-470,
+491-660); underneath it only forwards device pointers and the current stream to
+the C ABI declared in ``include/lplb_hip.h``.
+
+There is no CPU or pure-PyTorch fallback: if the shared library is missing or a
+tensor is not on a GPU, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from pathlib import Path
+
+import torch
+
+_PKG = Path(__file__).resolve().parent
+LIB_PATH = _PKG / "liblplb_hip.so"
+ABI_VERSION = 1
+
+STEP_REFERENCE_WINDOW = 0
+STEP_FULL_MAX = 1
+REFERENCE_STEPS = 5
+
+_lib: ctypes.CDLL | None = None
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+
+_SIGNATURES = {
+    "lplb_abi_version": (_i, []),
+    "lplb_last_error": (ctypes.c_char_p, []),
+    "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
+    "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+}
+
+
+def build(verbose: bool = False) -> Path:
+    """Compile the HIP library for gfx950 with the Makefile in ``csrc/``."""
+    proc = subprocess.run(["make", "-C", str(_PKG / "csrc"), "-B", "-j4"], capture_output=True, text=True)
+    if verbose or proc.returncode != 0:
+        print(proc.stdout)
+        print(proc.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError("building liblplb_hip.so failed")
+    return LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C {_PKG / 'csrc'}` "
+            "(hipcc, --offload-arch=gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.lplb_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"liblplb_hip.so has ABI {lib.lplb_abi_version()}, expected {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def exported_symbols() -> list[str]:
+    return list(_SIGNATURES)
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(f"lplb_hip error {rc}: {load().lplb_last_error().decode()}")
+
+
+def _require(cond: bool, what: str) -> None:
+    if not cond:
+        raise RuntimeError(f"LPLB assertion failed: {what}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class CompiledSolver:
+    """Launches the three planning kernels for one (n_group, G, D, P, C) shape."""
+
+    def __init__(self, n_group: int, group_size: int, dup_per_rank: int, n_local_experts: int,
+                 n_combined_experts: int) -> None:
+        self.lib = load()
+        self.n_group = n_group
+        self.group_size = group_size
+        self.dup_per_rank = dup_per_rank
+        self.n_local_experts = n_local_experts
+        self.n_combined_experts = n_combined_experts
+        # csrc/plugin.cpp:464-466
+        self.n_experts = (n_local_experts - dup_per_rank * n_combined_experts) * group_size * n_group
+        self.step_rule = STEP_REFERENCE_WINDOW
+        self.n_steps = REFERENCE_STEPS
+
+    # -- csrc/plugin.cpp:491-578 -------------------------------------------------
+    def solve(self, local_workload: torch.Tensor, r2o: torch.Tensor, phy2log: torch.Tensor,
+              avail_num: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        _require(local_workload.is_cuda, "local_workload on a GPU")
+        _require(local_workload.dim() == 3, "local_workload.dim() == 3")
+        n_group = local_workload.size(0)
+        _require(self.group_size == local_workload.size(1), "group_size == local_workload.size(1)")
+        n_logical_per_rank = local_workload.size(2)
+        n_pes = n_group * self.group_size
+        _require(local_workload.dtype == torch.int32, "local_workload.dtype == int32")
+        _require(local_workload.is_contiguous(), "local_workload.is_contiguous()")
+        _require(r2o.dim() == 2 and r2o.size(0) == self.group_size and r2o.size(1) == self.dup_per_rank,
+                 "r2o is [group_size, dup_per_rank]")
+        _require(r2o.dtype == torch.int32, "r2o.dtype == int32")
+        _require(phy2log.dim() == 1 and phy2log.size(0) % n_pes == 0, "phy2log is 1-D, a multiple of the EP size")
+        _require(phy2log.dtype == torch.int32, "phy2log.dtype == int32")
+        n_physical_per_rank = phy2log.size(0) // n_pes
+        _require((n_physical_per_rank - n_logical_per_rank) % self.dup_per_rank == 0,
+                 "replicas per rank divisible by dup_per_rank")
+        n_per_var = (n_physical_per_rank - n_logical_per_rank) // self.dup_per_rank
+        n_fixed = n_logical_per_rank - self.dup_per_rank * n_per_var
+        _require(avail_num.numel() == 1, "avail_num.numel() == 1")
+        _require(avail_num.dtype == torch.int32, "avail_num.dtype == int32")
+        _require(r2o.is_cuda and phy2log.is_cuda and avail_num.is_cuda, "all tensors on the GPU")
+        r2o = r2o.contiguous()
+        phy2log = phy2log.contiguous()
+        avail_num = avail_num if avail_num.is_contiguous() else avail_num.contiguous()
+
+        global_workload = torch.empty_like(local_workload, dtype=torch.float32)
+        result = torch.empty((n_group, self.group_size, self.dup_per_rank), dtype=torch.float32,
+                             device=local_workload.device)
+        _check(self.lib.lplb_solve(local_workload.data_ptr(), global_workload.data_ptr(), r2o.data_ptr(),
+                                   phy2log.data_ptr(), n_group, self.group_size, self.dup_per_rank,
+                                   n_per_var, n_fixed, avail_num.data_ptr(), result.data_ptr(),
+                                   self.step_rule, self.n_steps, _stream(local_workload)))
+        return result, global_workload
+
+    def solve_batched(self, workloads: torch.Tensor, r2o: torch.Tensor, phy2log: torch.Tensor,
+                      avail_num: torch.Tensor, want_global: bool = False):
+        """workloads int32 [n_instances, n_group, G, L] -> result fp32 [n_instances, n_group, G, D]."""
+        _require(workloads.is_cuda and workloads.dim() == 4 and workloads.dtype == torch.int32
+                 and workloads.is_contiguous(), "workloads is a contiguous int32 [N, n_group, G, L] GPU tensor")
+        n_inst, n_group, g, n_logical_per_rank = workloads.shape
+        _require(g == self.group_size, "group_size == workloads.size(2)")
+        n_pes = n_group * g
+        _require(phy2log.dtype == torch.int32 and phy2log.dim() == 1 and phy2log.size(0) % n_pes == 0,
+                 "phy2log is int32, 1-D, a multiple of the EP size")
+        _require(r2o.dtype == torch.int32 and tuple(r2o.shape) == (g, self.dup_per_rank), "r2o is int32 [G, D]")
+        _require(avail_num.numel() == 1 and avail_num.dtype == torch.int32, "avail_num is one int32")
+        n_per_var = (phy2log.size(0) // n_pes - n_logical_per_rank) // self.dup_per_rank
+        n_fixed = n_logical_per_rank - self.dup_per_rank * n_per_var
+        result = torch.empty((n_inst, n_group, g, self.dup_per_rank), dtype=torch.float32, device=workloads.device)
+        gw = torch.empty_like(workloads, dtype=torch.float32) if want_global else None
+        _check(self.lib.lplb_solve_batched(workloads.data_ptr(), gw.data_ptr() if want_global else None,
+                                           r2o.contiguous().data_ptr(), phy2log.contiguous().data_ptr(),
+                                           n_inst, n_group, g, self.dup_per_rank, n_per_var, n_fixed,
+                                           avail_num.data_ptr(), result.data_ptr(), self.step_rule,
+                                           self.n_steps, _stream(workloads)))
+        return (result, gw) if want_global else result
+
+    # -- csrc/plugin.cpp:580-600 -------------------------------------------------
+    def count_idx(self, idx: torch.Tensor, n_sms: int, block_dim: int = 256) -> tuple[torch.Tensor, torch.Tensor]:
+        _require(idx.dtype == torch.int64, "idx.dtype == int64")
+        _require(idx.is_cuda, "idx.device().is_cuda()")
+        _require(idx.is_contiguous(), "idx.is_contiguous()")
+        _require(block_dim == 256, "slices are aligned to 256 indices")
+        out = torch.empty((n_sms, self.n_experts), dtype=torch.int32, device=idx.device)
+        _check(self.lib.lplb_count_idx(idx.data_ptr(), idx.numel(), self.n_experts, n_sms, out.data_ptr(),
+                                       _stream(idx)))
+        return out[-1], out
+
+    # -- csrc/plugin.cpp:602-660 -------------------------------------------------
+    def map_idx(self, mapping_idx: torch.Tensor, o_weight: torch.Tensor, local_workload_split_by_sm: torch.Tensor,
+                o2r: torch.Tensor, phy2log: torch.Tensor, n_sms: int, block_dim: int = 256) -> torch.Tensor:
+        _require(mapping_idx.dtype == torch.int64, "mapping_idx.dtype == int64")
+        _require(mapping_idx.is_cuda, "mapping_idx.device().is_cuda()")
+        _require(mapping_idx.is_contiguous(), "mapping_idx.is_contiguous()")
+        _require(o_weight.dtype == torch.float32, "o_weight.dtype == float32")
+        _require(o_weight.is_cuda and o_weight.is_contiguous(), "o_weight is a contiguous GPU tensor")
+        _require(o_weight.dim() == 3 and tuple(o_weight.shape) == (self.n_group, self.group_size, self.dup_per_rank),
+                 "o_weight is [n_group, group_size, dup_per_rank]")
+        _require(o2r.dtype == torch.int32 and o2r.is_cuda and o2r.is_contiguous(), "o2r is a contiguous int32 GPU tensor")
+        _require(o2r.dim() == 2 and tuple(o2r.shape) == (self.group_size, self.dup_per_rank),
+                 "o2r is [group_size, dup_per_rank]")
+        _require(phy2log.dtype == torch.int32 and phy2log.is_cuda and phy2log.is_contiguous(),
+                 "phy2log is a contiguous int32 GPU tensor")
+        _require(phy2log.dim() == 1 and phy2log.size(0) == self.group_size * self.n_group * self.n_local_experts,
+                 "phy2log.size(0) == group_size * n_group * n_local_experts")
+        by_sm = local_workload_split_by_sm
+        _require(by_sm.dtype == torch.int32 and by_sm.is_cuda and by_sm.is_contiguous()
+                 and tuple(by_sm.shape) == (n_sms, self.n_experts),
+                 "local_workload_split_by_sm is a contiguous int32 [n_sms, n_experts] GPU tensor")
+        _require(block_dim == 256, "slices are aligned to 256 indices")
+        out = torch.empty_like(mapping_idx)
+        _check(self.lib.lplb_map_idx(mapping_idx.data_ptr(), o_weight.data_ptr(), by_sm.data_ptr(), o2r.data_ptr(),
+                                     phy2log.data_ptr(), mapping_idx.numel(), self.n_group, self.group_size,
+                                     self.dup_per_rank, self.n_combined_experts, self.n_local_experts, n_sms,
+                                     out.data_ptr(), _stream(mapping_idx)))
+        return out

@@ -1,0 +1,83 @@
+// Shared host/device helpers of the planning kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lplb_hip.h"
+
+namespace lplb {
+
+constexpr int kWave = 64;
+// Slice boundaries are aligned to this many indices whatever the workgroup
+// size is; it is part of the observable slice partition (minilp.cu:404-408
+// is called with the reference's fixed block size of 256).
+constexpr int kSliceAlign = 256;
+
+// Records a message for lplb_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define LPLB_REQUIRE(cond, code, ...)                                          \
+  do {                                                                         \
+    if (!(cond))                                                               \
+      return ::lplb::fail((code), __VA_ARGS__);                                \
+  } while (0)
+
+#define LPLB_HIP_TRY(expr)                                                     \
+  do {                                                                         \
+    hipError_t e_ = (expr);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return ::lplb::fail(LPLB_EHIP, "%s failed: %s", #expr,                   \
+                          hipGetErrorString(e_));                              \
+  } while (0)
+
+// Length of one slice: ceil(n / parts) rounded up to kSliceAlign.
+__host__ __device__ inline int64_t slice_len(int64_t n, int parts) {
+  int64_t per = (n + parts - 1) / parts;
+  return (per + kSliceAlign - 1) / kSliceAlign * kSliceAlign;
+}
+
+__host__ __device__ inline int64_t slice_begin(int64_t n, int64_t per, int p) {
+  int64_t v = per * p;
+  return v < n ? v : n;
+}
+
+// ---- wave64 primitives -----------------------------------------------------
+
+__device__ inline int lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+template <typename T> __device__ inline T bpermute(T v, int src_lane) {
+  static_assert(sizeof(T) == 4, "32-bit values only");
+  int r = __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v));
+  return __builtin_bit_cast(T, r);
+}
+
+// Value of `v` in lane `src` (wave-uniform, compile-time or scalar `src`).
+__device__ inline float readlane(float v, int src) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
+}
+__device__ inline double readlane(double v, int src) {
+  int2 p = __builtin_bit_cast(int2, v);
+  p.x = __builtin_amdgcn_readlane(p.x, src);
+  p.y = __builtin_amdgcn_readlane(p.y, src);
+  return __builtin_bit_cast(double, p);
+}
+
+// Butterfly reductions; every lane ends with the result.
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1)
+    v += bpermute(v, lane_id() ^ off);
+  return v;
+}
+// fmaxf semantics: a NaN operand is ignored unless both are NaN.
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1)
+    v = fmaxf(v, bpermute(v, lane_id() ^ off));
+  return v;
+}
+
+} // namespace lplb

@@ -1,0 +1,158 @@
+"""Per-batch token planner for expert-parallel MoE on MI355X.
+
+``Planner`` is a drop-in for the reference's ``lplb.Planner`` (lplb/planner.py:38-266):
+same constructor, attributes and methods, same tensors in and out.  ``run`` chains
+three HIP launches on the current stream -- histogram, LP solve, redirect -- without
+any host synchronisation.
+"""
+from __future__ import annotations
+
+import functools
+
+import numpy as np
+import torch
+
+from ._native import CompiledSolver
+from .mapping import build_redundancy_mapping
+
+
+@functools.lru_cache(maxsize=None)
+def _get_solver(n_group: int, group_size: int, dup_per_rank: int, n_local_experts: int,
+                n_combined_experts: int) -> CompiledSolver:
+    return CompiledSolver(n_group, group_size, dup_per_rank, n_local_experts, n_combined_experts)
+
+
+class Planner:
+    def __init__(
+        self,
+        redundant_to_original: torch.Tensor,
+        n_routed_experts: int,
+        n_logical_routed_experts: int,
+        ep_size: int | None = None,
+        group: "torch.distributed.ProcessGroup | None" = None,
+        *,
+        device: str | torch.device = "cuda",
+        gpus_per_node: int | None = None,
+    ) -> None:
+        """
+        :param redundant_to_original: [group_size, num_redundants]; entry (i, d) is the group-rank
+            whose d-th replicated expert set is copied into replica slot d of group-rank i.  Every
+            column must be a permutation, so that each replica joins exactly two ranks.  A rank may
+            hold a multiple of ``num_redundants`` replicas; they are pooled per slot for the LP.
+        :param n_routed_experts: physical routed experts (originals + replicas) over all ranks.
+        :param n_logical_routed_experts: logical routed experts.
+        :param ep_size: number of EP ranks; defaults to ``group.size()``.
+        :param group: EP process group; ``None`` means the workload handed to ``solve_probs`` is
+            already global and no reduction is done.
+        :param device: where the planner's tensors live.  Everything except the redundancy-mapping
+            bookkeeping needs a GPU.
+        :param gpus_per_node: GPUs per node for EPLB's node-aware packing; defaults to the number
+            of visible GPUs (lplb/planner.py:132).
+        """
+        self.device = torch.device(device)
+        r2o = torch.as_tensor(redundant_to_original)
+        assert r2o.dim() == 2, "redundant_to_original must be [group_size, num_redundants]"
+        self.r2o = r2o.to(dtype=torch.int32, device=self.device).contiguous()
+        self.o2r = self.r2o.argsort(dim=0).to(torch.int32).contiguous()
+        self.group_size, self.num_redundants = int(r2o.shape[0]), int(r2o.shape[1])
+        self._r2o_host = self.r2o.cpu().numpy()
+
+        self.n_routed_experts = n_routed_experts
+        self.n_logical_routed_experts = n_logical_routed_experts
+        if ep_size is not None:
+            self.ep_size = ep_size
+        else:
+            assert group is not None, "ep_size must be provided when group is None"
+            self.ep_size = group.size()
+        self.n_group = self.ep_size // self.group_size
+
+        self.n_local_routed_experts = self.n_routed_experts // self.ep_size
+        self.n_local_logical_routed_experts = self.n_logical_routed_experts // self.ep_size
+        self.combined_redundant_experts = (
+            self.n_local_routed_experts - self.n_local_logical_routed_experts
+        ) // self.num_redundants
+
+        if gpus_per_node is None:
+            gpus_per_node = torch.cuda.device_count() or 1
+        self.gpus_per_node = gpus_per_node
+
+        self.phy2log: torch.Tensor
+        self.update_redundancy_mapping()
+
+        self.ep_group = group
+        self.deep_ep_initialized = False
+        self._solver: CompiledSolver | None = None
+
+    @property
+    def solver(self) -> CompiledSolver:
+        if self._solver is None:
+            if self.device.type != "cuda":
+                raise RuntimeError("the planning kernels need a GPU: construct the Planner with device='cuda'")
+            self._solver = _get_solver(self.n_group, self.group_size, self.num_redundants,
+                                       self.n_local_routed_experts, self.combined_redundant_experts)
+        return self._solver
+
+    def init_from_deep_ep(self, buffer) -> None:
+        """The reference can take its workload reduction from a DeepEP buffer's NVSHMEM team
+        (lplb/planner.py:104-113).  There is no such transport here."""
+        raise NotImplementedError(
+            "in-kernel workload reduction through a DeepEP buffer is not available; "
+            "pass `group` to reduce with torch.distributed, or hand solve_probs a global workload")
+
+    def update_redundancy_mapping(
+        self, workload: torch.Tensor | None = None
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Choose which experts get replicas (lplb/planner.py:115-182).
+
+        :param workload: per-logical-expert history; ``None`` keeps experts in index order.
+        :return: ``(phy2log [n_routed], log2phy [n_logical, 2], logcnt [n_logical])``, int32.
+        """
+        host = None if workload is None else workload.detach().cpu().numpy()
+        phy2log, log2phy, logcnt = build_redundancy_mapping(
+            self._r2o_host, self.ep_size, self.n_logical_routed_experts, self.n_routed_experts,
+            host, n_nodes=max(1, self.ep_size // self.gpus_per_node))
+        to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(self.device)  # noqa: E731
+        self.phy2log = to_dev(phy2log)
+        return self.phy2log, to_dev(log2phy), to_dev(logcnt)
+
+    def count_workload(self, idx: torch.Tensor, n_sms: int) -> tuple[torch.Tensor, torch.Tensor]:
+        """Histogram of ``idx`` (values in [-1, n_logical), -1 ignored) over ``n_sms`` slices.
+
+        :return: (counts [n_logical], running counts per slice [n_sms, n_logical]), int32.
+        """
+        return self.solver.count_idx(idx, n_sms, 256)
+
+    def solve_probs(self, workload: torch.Tensor, avail_counter: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """Solve the balancing LP of every EP group.
+
+        :param workload: int32 per-logical-expert counts (numel = n_logical).
+        :param avail_counter: int32, numel 1; incremented once per feasible group.
+        :return: (share kept on the original rank, fp32 [n_group, group_size, num_redundants];
+                  normalised global workload, fp32 [n_group, group_size, L]).
+        """
+        workload = workload.view(self.n_group, self.group_size, self.n_local_logical_routed_experts)
+        if self.ep_group is not None and not self.deep_ep_initialized:
+            workload = workload.clone()
+            torch.distributed.all_reduce(workload, group=self.ep_group)
+        return self.solver.solve(workload, self.r2o, self.phy2log, avail_counter)
+
+    def weighted_select_target(self, idx: torch.Tensor, o_weight: torch.Tensor,
+                               local_workload_by_sm: torch.Tensor, n_sms: int) -> torch.Tensor:
+        """Map logical expert ids to physical ones according to ``o_weight``.
+
+        :return: int64, same shape as ``idx``, values in [-1, n_routed_experts).
+        """
+        return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256)
+
+    def run(self, idx: torch.Tensor, avail_counter: torch.Tensor, n_sms: int | None = None) -> torch.Tensor:
+        """Assign a physical expert to every selected logical expert.
+
+        :param idx: int64 logical expert ids, any shape, contiguous, values in [-1, n_logical).
+        :param avail_counter: int32 tensor with one element, counts feasible LP solves.
+        :param n_sms: number of slices / workgroups; defaults to the GPU's compute-unit count.
+        """
+        if n_sms is None:
+            n_sms = torch.cuda.get_device_properties(idx.device).multi_processor_count
+        local_workload, local_workload_by_sm = self.count_workload(idx, n_sms)
+        o_weight, _global_workload = self.solve_probs(local_workload, avail_counter)
+        return self.weighted_select_target(idx, o_weight, local_workload_by_sm, n_sms)

@@ -1,0 +1,267 @@
+"""HIP path vs the CPU oracle on the same seeded inputs (needs an MI355X).
+
+Bars: histogram, prefix and redirect are bit-exact; the LP result must give an
+objective (max rank load) within 1e-3 relative and edge flows within 1e-4 of the
+total token count of the oracle's, which follows the reference's fp32 arithmetic.
+"""
+import numpy as np
+import pytest
+import torch
+
+from lplb_amd import Planner, synth
+from lplb_amd._native import CompiledSolver
+from oracle import oracle
+from tests.helpers import CASE_SEED, REFERENCE_SOLVE_CASES, Shape, reference_style_case
+
+pytestmark = pytest.mark.gpu
+
+OBJ_RTOL = 1e-3      # objective, relative
+FLOW_TOL = 1e-4      # edge flows, relative to the total token count
+
+
+def dev(a, cuda, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.to(cuda)
+
+
+def solver_for(s: Shape) -> CompiledSolver:
+    return CompiledSolver(s.n_group, s.G, s.D, s.P, s.C)
+
+
+# ----------------------------------------------------------------- histogram
+@pytest.mark.parametrize("n,n_experts,n_sms", [
+    (4096 * 8, 256, 256), (65536, 256, 100), (0, 256, 8), (1, 32, 4), (255, 32, 3), (257, 32, 3),
+    (1000003, 256, 256), (70001, 1000, 37), (65536, 256, 1), (8192 * 8, 256, 304),
+])
+def test_count_idx_matches_oracle(cuda, n, n_experts, n_sms):
+    rng = np.random.default_rng(n + n_experts + n_sms)
+    idx = rng.integers(-1, n_experts, size=n, dtype=np.int64)
+    solver = CompiledSolver(1, 1, 1, n_experts + 1, 1)   # n_experts logical experts
+    assert solver.n_experts == n_experts
+    total, by_sm = solver.count_idx(dev(idx, cuda), n_sms)
+    torch.cuda.synchronize()
+    want = oracle.count_idx(idx, n_experts, n_sms)
+    assert by_sm.shape == (n_sms, n_experts) and by_sm.dtype == torch.int32
+    np.testing.assert_array_equal(by_sm.cpu().numpy(), want)
+    # properties the reference's own test checks (tests/test_idx_processing.py:36-48)
+    assert total.shape == (n_experts,)
+    assert int(total.min()) >= 0
+    assert int(total.sum()) == int((idx != -1).sum())
+    np.testing.assert_array_equal(total.cpu().numpy(), np.bincount(idx[idx >= 0], minlength=n_experts))
+
+
+# ------------------------------------------------------------------ redirect
+def _random_weights(shape: Shape, rng):
+    w = rng.standard_normal((shape.n_group, shape.G, shape.D)) / 3 + 0.5
+    return np.clip(w, 0, 1).astype(np.float32)
+
+
+@pytest.mark.parametrize("case", ["cube8_ep32", "cube8_ep32_c2", "ring8_ep32", "hypercube16", "torus8x4"])
+@pytest.mark.parametrize("n,n_sms", [(65536, 256), (4099, 7), (300, 256), (1 << 20, 256)])
+def test_map_idx_matches_oracle(cuda, case, n, n_sms):
+    name, r2o, nl, ep, red, reorder, _ = next(c for c in REFERENCE_SOLVE_CASES if c[0] == case)
+    shape, _, phy2log, log2phy, _ = reference_style_case(r2o, nl, ep, red, True, seed=7)
+    rng = np.random.default_rng(n * 31 + n_sms)
+    idx = rng.integers(-1, nl, size=n, dtype=np.int64)
+    o_weight = _random_weights(shape, rng)
+    solver = solver_for(shape)
+    d_idx = dev(idx, cuda)
+    _, by_sm = solver.count_idx(d_idx, n_sms)
+    out = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+    np.testing.assert_array_equal(got, want)
+    # reference test's properties (tests/test_idx_processing.py:88-98)
+    assert got.min() >= -1 and got.max() < shape.n_physical
+    assert np.array_equal(got == -1, idx == -1)
+    padded = np.concatenate([np.full((1, 2), -1, np.int32), log2phy])
+    assert np.all((got == padded[idx + 1, 0]) | (got == padded[idx + 1, 1]))
+    # conservation
+    assert np.bincount(got[got >= 0], minlength=shape.n_physical).sum() == (idx != -1).sum()
+
+
+def test_map_idx_is_independent_of_slicing(cuda):
+    shape, _, phy2log, _, _ = reference_style_case(*REFERENCE_SOLVE_CASES[0][1:6], seed=3)
+    rng = np.random.default_rng(5)
+    idx = rng.integers(-1, shape.n_logical, size=50000, dtype=np.int64)
+    o_weight = _random_weights(shape, rng)
+    solver = solver_for(shape)
+    outs = []
+    for n_sms in (1, 13, 256):
+        d_idx = dev(idx, cuda)
+        _, by_sm = solver.count_idx(d_idx, n_sms)
+        outs.append(solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda),
+                                   n_sms).cpu().numpy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_map_idx_extreme_weights(cuda):
+    """o_weight outside [0, 1] and NaN: everything to the replica / original, nothing lost."""
+    shape, _, phy2log, _, _ = reference_style_case(*REFERENCE_SOLVE_CASES[0][1:6], seed=3)
+    rng = np.random.default_rng(11)
+    idx = rng.integers(-1, shape.n_logical, size=20000, dtype=np.int64)
+    o_weight = rng.choice(np.array([-1.5, 0.0, 0.3, 1.0, 2.5, np.nan, 1e30, -1e30], np.float32),
+                          size=(shape.n_group, shape.G, shape.D))
+    solver = solver_for(shape)
+    d_idx = dev(idx, cuda)
+    _, by_sm = solver.count_idx(d_idx, 64)
+    got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 64).cpu().numpy()
+    want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+    np.testing.assert_array_equal(got, want)
+
+
+# -------------------------------------------------------------------- solver
+def _compare_solve(shape, phy2log, workload, res, gw, avail, step_rule=0, n_steps=5):
+    o_res, o_gw, o_avail = oracle.solve(workload, shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed,
+                                        step_rule=step_rule, n_steps=n_steps)
+    o64, _, _ = oracle.solve(workload, shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed,
+                             step_rule=step_rule, n_steps=n_steps, precision=64)
+    np.testing.assert_array_equal(gw.reshape(-1), o_gw)          # fp32 divide, bit-exact
+    assert avail == o_avail
+    total = float(np.sum(workload, dtype=np.float64))
+    args = (shape.r2o, phy2log, shape.n_group, shape.C)
+    out = {}
+    for tag, ref in (("f32", o_res), ("f64", o64)):
+        flow = np.abs(oracle.edge_flows(workload, res, *args) - oracle.edge_flows(workload, ref, *args)).max() / total
+        obj_ref = oracle.rank_loads(workload, ref, *args).max(axis=1)
+        obj = oracle.rank_loads(workload, res, *args).max(axis=1)
+        out[tag] = (flow, (np.abs(obj - obj_ref) / obj_ref).max(), np.abs(res - ref).max())
+    print(f"  flow/obj/p diff vs oracle f32 {out['f32']}, vs f64 {out['f64']}")
+    assert out["f32"][0] <= FLOW_TOL and out["f32"][1] <= OBJ_RTOL
+    return out
+
+
+@pytest.mark.parametrize("case", REFERENCE_SOLVE_CASES, ids=[c[0] for c in REFERENCE_SOLVE_CASES])
+def test_solve_reference_cases(cuda, case):
+    """The reference's solver test (tests/test_solve.py:13-89) plus parity with the oracle."""
+    name, r2o, nl, ep, red, reorder, tol = case
+    shape, hist, phy2log, _, workload = reference_style_case(r2o, nl, ep, red, reorder, seed=CASE_SEED[name])
+    planner = Planner(torch.from_numpy(shape.r2o), shape.n_physical, nl, ep, gpus_per_node=8)
+    got_p2l, _, _ = planner.update_redundancy_mapping(None if hist is None else torch.from_numpy(hist))
+    np.testing.assert_array_equal(got_p2l.cpu().numpy(), phy2log)
+    avail = torch.zeros((), dtype=torch.int32, device=cuda)
+    probs, gw = planner.solve_probs(dev(workload, cuda), avail)
+    torch.cuda.synchronize()
+    assert probs.shape == (shape.n_group, shape.G, shape.D) and probs.dtype == torch.float32
+    assert int(avail) == planner.n_group
+    res = probs.cpu().numpy()
+    loads = oracle.rank_loads(workload, res, shape.r2o, phy2log, shape.n_group, shape.C)
+    balance = loads.max() / loads.mean()
+    print(f"{name}: balance {balance:.4f} (tolerance {tol})")
+    assert balance < tol
+    _compare_solve(shape, phy2log, workload, res, gw.cpu().numpy(), int(avail))
+
+
+@pytest.mark.parametrize("cfg", ["cpu_ref_ep8", "v3_ep8_cube", "ep16_hypercube", "ep32_torus"])
+@pytest.mark.parametrize("step_rule", [0, 1])
+def test_solve_benchmark_configs(cuda, cfg, step_rule):
+    inp = synth.make_inputs(cfg, tokens=64)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    solver = solver_for(shape)
+    solver.step_rule = step_rule
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    wl = dev(inp.global_counts.reshape(shape.n_group, shape.G, shape.L), cuda)
+    res, gw = solver.solve(wl, dev(shape.r2o, cuda), dev(inp.phy2log, cuda), avail)
+    torch.cuda.synchronize()
+    _compare_solve(shape, inp.phy2log, inp.global_counts, res.cpu().numpy(), gw.cpu().numpy(), int(avail[0]),
+                   step_rule=step_rule)
+
+
+def test_solve_fallback_and_counter(cuda):
+    """Infeasible / degenerate LPs give 0.5 everywhere and leave the counter alone;
+    the counter accumulates across calls (minilp.cu:379-400)."""
+    shape, _, phy2log, _, workload = reference_style_case(*REFERENCE_SOLVE_CASES[0][1:6])
+    solver = solver_for(shape)
+    args = (dev(shape.r2o, cuda), dev(phy2log, cuda))
+    avail = torch.full((1,), 7, dtype=torch.int32, device=cuda)
+    zero = torch.zeros((shape.n_group, shape.G, shape.L), dtype=torch.int32, device=cuda)
+    res, gw = solver.solve(zero, *args, avail)
+    assert torch.all(res == 0.5) and int(avail[0]) == 7
+    assert torch.isnan(gw).all()
+    solver.n_steps = 1          # one step cannot pass the feasibility test
+    res, _ = solver.solve(dev(workload.reshape(zero.shape), cuda), *args, avail)
+    assert torch.all(res == 0.5) and int(avail[0]) == 7
+    solver.n_steps = 5
+    for k in (1, 2):
+        res, _ = solver.solve(dev(workload.reshape(zero.shape), cuda), *args, avail)
+        assert int(avail[0]) == 7 + k * shape.n_group
+    o_res, _, _ = oracle.solve(workload, shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed, n_steps=1)
+    assert np.all(o_res == 0.5)
+
+
+def test_solve_batched_matches_single(cuda):
+    inp = synth.make_inputs("v3_ep8_cube", tokens=8)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    counts = synth.sweep_counts(64)
+    solver = solver_for(shape)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    r2o, p2l = dev(shape.r2o, cuda), dev(inp.phy2log, cuda)
+    batched, gws = solver.solve_batched(dev(counts.reshape(64, 1, shape.G, shape.L), cuda), r2o, p2l, avail,
+                                        want_global=True)
+    assert int(avail[0]) == 64
+    for i in (0, 17, 63):
+        single, gw = solver.solve(dev(counts[i].reshape(1, shape.G, shape.L), cuda), r2o, p2l, avail)
+        assert torch.equal(single[0], batched[i, 0]) and torch.equal(gw, gws[i])
+        _compare_solve(shape, inp.phy2log, counts[i], batched[i].cpu().numpy(), gws[i].cpu().numpy(), 1)
+
+
+# ------------------------------------------------------------------ whole plan
+@pytest.mark.parametrize("cfg,mask", [("cpu_ref_ep8", 0.0), ("v3_ep8_cube", 0.05), ("ep16_hypercube", 0.05),
+                                      ("ep32_torus", 0.0)])
+def test_run_matches_oracle_chain(cuda, cfg, mask):
+    inp = synth.make_inputs(cfg, mask_fraction=mask)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    planner.phy2log = dev(inp.phy2log, cuda)
+    n_sms = 256
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    d_idx = dev(inp.indices, cuda)
+    out = planner.run(d_idx, avail, n_sms)
+    torch.cuda.synchronize()
+    assert out.shape == d_idx.shape and out.dtype == torch.int64
+    # the same chain on the CPU, fed with the GPU's own flow vector for the redirect
+    by_sm = oracle.count_idx(inp.indices, c.n_logical, n_sms)
+    local, by_sm_gpu = planner.count_workload(d_idx, n_sms)
+    np.testing.assert_array_equal(by_sm_gpu.cpu().numpy(), by_sm)
+    o_weight, gw = planner.solve_probs(local, torch.zeros(1, dtype=torch.int32, device=cuda))
+    _compare_solve(shape, inp.phy2log, by_sm[-1], o_weight.cpu().numpy(), gw.cpu().numpy(), int(avail[0]))
+    want = oracle.map_idx(inp.indices, o_weight.cpu().numpy(), by_sm, shape.o2r, inp.phy2log, shape.n_group,
+                          shape.C, shape.P)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
+def test_redirect_full_size_sweep(cuda):
+    """[262144 x 8] indices: bit-exact against the oracle, exact split counts, conservation."""
+    inp = synth.make_inputs("sweep_redirect")
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    solver = solver_for(shape)
+    d_idx = dev(inp.indices, cuda)
+    total, by_sm = solver.count_idx(d_idx, 256)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    o_weight, _ = solver.solve(total.view(1, shape.G, shape.L), dev(shape.r2o, cuda), dev(inp.phy2log, cuda), avail)
+    out = solver.map_idx(d_idx, o_weight, by_sm, dev(shape.o2r, cuda), dev(inp.phy2log, cuda), 256)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = oracle.map_idx(inp.indices, o_weight.cpu().numpy(), by_sm.cpu().numpy(), shape.o2r, inp.phy2log, 1,
+                          shape.C, shape.P)
+    np.testing.assert_array_equal(got, want)
+    # exact number of tokens kept on the original: clamp(trunc(w * total), 0, total) when 499 does not divide total
+    tot = total.cpu().numpy().astype(np.int64)
+    phys = np.bincount(got.reshape(-1), minlength=c.n_physical)
+    assert phys.sum() == inp.indices.size
+    w = o_weight.cpu().numpy().reshape(shape.G, shape.D)
+    p2l = inp.phy2log.reshape(c.ep_size, shape.P)
+    for rank in range(c.ep_size):
+        for slot in range(shape.C * shape.D):
+            e = p2l[rank, slot]
+            if tot[e] % 499 == 0:
+                continue
+            keep = int(np.clip(np.trunc(np.float32(w[rank, slot % shape.D]) * np.float32(tot[e])), 0, tot[e]))
+            assert phys[rank * shape.P + slot] == keep, (rank, slot)
