@@ -1,0 +1,322 @@
+"""Benchmark of the per-batch planning path on one MI355X.
+
+One step = one plan of the DeepSeek-V3-shaped EP8 cube configuration: histogram of
+this GPU's [8192 x 8] routing indices, LP solve on the global per-expert counts,
+logical->physical redirect.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is the p50 GPU time per plan in microseconds, from
+HIP events recorded between plans on the stream the kernels run on.  The line also
+carries
+  roofline      redirect kernel at the sweep shape [262144 x 8] against the HBM peak;
+                algorithmic traffic is 16 bytes per index (int64 in, int64 out);
+  cpu_baseline  the scalar C restatement of the reference algorithm (oracle/), timed
+                on this host on a bounded sample of the same plans;
+  extras        p99, solve-only latency, batched plans/s, redirect tokens/s, ...
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+REDIRECT_BYTES_PER_INDEX = 16
+HISTOGRAM_BYTES_PER_INDEX = 8
+
+
+def pct(a, q):
+    return float(np.percentile(np.asarray(a, dtype=np.float64), q))
+
+
+def event_times_us(fn, n, warmup, torch):
+    """Runs fn() n times back to back; returns GPU microseconds between consecutive events."""
+    for _ in range(warmup):
+        fn()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for i in range(n):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    return np.array([ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(n)])
+
+
+class KernelTimer:
+    """Times single kernels of the library by their own begin/end timestamps: the library
+    records them into a pair of HIP events armed with lplb_time_next_launch()."""
+
+    def __init__(self, lib, n):
+        import ctypes
+        self.ct = ctypes
+        self.lib = lib
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        self.pairs = []
+        for _ in range(n):
+            a, b = ctypes.c_void_p(), ctypes.c_void_p()
+            assert self.hip.hipEventCreate(ctypes.byref(a)) == 0 and self.hip.hipEventCreate(ctypes.byref(b)) == 0
+            self.pairs.append((a, b))
+        self.used = 0
+
+    def arm(self):
+        a, b = self.pairs[self.used]
+        self.used += 1
+        self.lib.lplb_time_next_launch(a, b)
+
+    def times_us(self, torch):
+        torch.cuda.synchronize()
+        out = []
+        for a, b in self.pairs[:self.used]:
+            ms = self.ct.c_float()
+            rc = self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b)
+            assert rc == 0, f"hipEventElapsedTime -> {rc}"
+            out.append(ms.value * 1e3)
+        self.used = 0
+        return np.array(out)
+
+    def close(self):
+        for a, b in self.pairs:
+            self.hip.hipEventDestroy(a)
+            self.hip.hipEventDestroy(b)
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--skip-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the plan; a run with --gpus > 1 is not supported "
+                 "(the path needs no collective: see DESIGN.md, sharding).")
+
+    import torch
+
+    from lplb_amd import synth
+    from lplb_amd._native import CompiledSolver, load
+    from oracle import oracle
+
+    load()  # no fallback: raises if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    props = torch.cuda.get_device_properties(dev)
+    n_sms = props.multi_processor_count
+
+    def to_dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    # ------------------------------------------------------------------ inputs
+    inp = synth.make_inputs("v3_ep8_cube")
+    cfg = inp.cfg
+    G, D = cfg.r2o.shape
+    L, P = cfg.n_logical // cfg.ep_size, cfg.n_physical // cfg.ep_size
+    C = (P - L) // D
+    n_fixed = L - C * D
+    o2r_host = np.argsort(cfg.r2o, axis=0, kind="stable").astype(np.int32)
+    solver = CompiledSolver(1, G, D, P, C)
+    r2o, o2r, phy2log = to_dev(cfg.r2o), to_dev(o2r_host), to_dev(inp.phy2log)
+    idx = to_dev(inp.indices)
+    counts = to_dev(inp.global_counts)
+    avail = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws: dict = {}
+
+    def plan():
+        out, o_w, by = solver.plan(idx, r2o, o2r, phy2log, avail, n_sms, global_counts=counts, workspace=ws)
+        ws["out"], ws["o_weight"], ws["by_sm"] = out, o_w, by
+
+    plan()
+    ws["global_workload"] = torch.empty(cfg.n_logical, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+
+    # ----------------------------------------------------------- timed region
+    for _ in range(args.warmup):
+        plan()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(args.steps):
+        plan()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per_plan_us = np.array([ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(args.steps)])
+    p50, p99 = pct(per_plan_us, 50), pct(per_plan_us, 99)
+    assert int(avail[0]) == args.warmup + args.steps + 1, "an LP failed its feasibility test"
+
+    extras: dict = {"p99_us_per_plan": round(p99, 2), "mean_us_per_plan": round(float(per_plan_us.mean()), 2),
+                    "compute_units": n_sms, "device": props.name}
+
+    # ------------------------------------------- roofline: redirect @ sweep shape
+    sweep = synth.make_inputs("sweep_redirect")
+    n_idx = sweep.indices.size
+    n_buf = 18                                   # 18 x (16 + 16) MiB > 512 MB of distinct lines
+    rng = np.random.default_rng(7)
+    flat = sweep.indices.reshape(-1)
+    bufs_in = [to_dev(np.roll(flat, int(rng.integers(0, n_idx)))) for _ in range(n_buf)]
+    bufs_out = [torch.empty_like(b) for b in bufs_in]
+    sweep_p2l = to_dev(sweep.phy2log)
+    tables = []
+    for b in bufs_in:
+        total, by = solver.count_idx(b, n_sms)
+        tables.append(by)
+    o_w, _ = solver.solve(tables[0][-1].view(1, G, L), r2o, sweep_p2l, avail)
+    lib = solver.lib
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def redirect(i):
+        rc = lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), tables[i].data_ptr(), o2r.data_ptr(),
+                              sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_sms, bufs_out[i].data_ptr(), stream)
+        assert rc == 0
+
+    reps = 20
+    for i in range(n_buf):
+        redirect(i)
+    timer = KernelTimer(lib, reps * n_buf)
+    torch.cuda.synchronize()
+    for _ in range(reps):
+        for i in range(n_buf):
+            timer.arm()
+            redirect(i)
+    red_us = timer.times_us(torch)
+    red_avg = float(red_us.mean())
+    alg_bytes = n_idx * REDIRECT_BYTES_PER_INDEX
+    achieved = alg_bytes / (red_avg * 1e-6) / 1e9
+    # the same bytes through a plain copy kernel: the practical ceiling on this box
+    for _ in range(reps):
+        for i in range(n_buf):
+            timer.arm()
+            assert lib.lplb_copy_calibration(bufs_in[i].data_ptr(), bufs_out[i].data_ptr(), n_idx, stream) == 0
+    copy_us = timer.times_us(torch)
+    copy_gbs = alg_bytes / (float(copy_us.mean()) * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "redirect_indices", "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64",
+                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
+                "p50_launch_us": round(pct(red_us, 50), 2), "distinct_buffer_pairs": n_buf,
+                "copy_kernel_GBs_same_bytes": round(copy_gbs, 1),
+                "frac_of_copy_kernel": round(achieved / copy_gbs, 4)}
+    extras["redirect_tokens_per_s"] = round(n_idx / (red_avg * 1e-6), 1)
+
+    if not args.skip_extras:
+        # histogram at the sweep shape (8 B per index)
+        def hist(i):
+            rc = lib.lplb_count_idx(bufs_in[i].data_ptr(), n_idx, cfg.n_logical, n_sms, tables[i].data_ptr(), stream)
+            assert rc == 0
+        k = [0]
+
+        def hist_next():
+            hist(k[0] % n_buf)
+            k[0] += 1
+        h_us = event_times_us(hist_next, 10 * n_buf, n_buf, torch)
+        extras["histogram_sweep_us"] = round(float(h_us.mean()), 2)
+        extras["histogram_sweep_GBs"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (float(h_us.mean()) * 1e-6) / 1e9, 1)
+
+        # kernels of the plan in isolation, at the plan's own shape
+        wl = counts.view(1, G, L)
+        gw = torch.empty(1, G, L, dtype=torch.float32, device=dev)
+        res = torch.empty(1, G, D, dtype=torch.float32, device=dev)
+
+        def solve_only():
+            lib.lplb_solve(wl.data_ptr(), gw.data_ptr(), r2o.data_ptr(), phy2log.data_ptr(), 1, G, D, C, n_fixed,
+                           avail.data_ptr(), res.data_ptr(), 0, 5, stream)
+        s_us = event_times_us(solve_only, 1000, 100, torch)
+        extras["solve_p50_us"] = round(pct(s_us, 50), 2)
+        extras["solve_p99_us"] = round(pct(s_us, 99), 2)
+
+        by_plan = ws["by_sm"]
+
+        def count_only():
+            lib.lplb_count_idx(idx.data_ptr(), idx.numel(), cfg.n_logical, n_sms, by_plan.data_ptr(), stream)
+
+        def map_only():
+            lib.lplb_map_idx(idx.data_ptr(), ws["o_weight"].data_ptr(), by_plan.data_ptr(), o2r.data_ptr(),
+                             phy2log.data_ptr(), idx.numel(), 1, G, D, C, P, n_sms, ws["out"].data_ptr(), stream)
+        extras["count_p50_us"] = round(pct(event_times_us(count_only, 1000, 100, torch), 50), 2)
+        extras["redirect_p50_us"] = round(pct(event_times_us(map_only, 1000, 100, torch), 50), 2)
+
+        # 2048 independent LP instances in one launch
+        sweep_wl = to_dev(synth.sweep_counts(2048).reshape(2048, 1, G, L))
+        results = torch.empty(2048, 1, G, D, dtype=torch.float32, device=dev)
+
+        def batched():
+            lib.lplb_solve_batched(sweep_wl.data_ptr(), None, r2o.data_ptr(), phy2log.data_ptr(), 2048, 1, G, D, C,
+                                   n_fixed, avail.data_ptr(), results.data_ptr(), 0, 5, stream)
+        b_us = event_times_us(batched, 100, 10, torch)
+        extras["batched_2048_solves_us"] = round(pct(b_us, 50), 2)
+        extras["batched_plans_per_s"] = round(2048 / (pct(b_us, 50) * 1e-6), 1)
+
+        # Planner.run through the Python API, wall clock with a device sync (host overhead included)
+        from lplb_amd import Planner
+        planner = Planner(torch.from_numpy(cfg.r2o), cfg.n_physical, cfg.n_logical, cfg.ep_size, device=dev)
+        planner.phy2log = phy2log
+        for _ in range(50):
+            planner.run(idx, avail, n_sms)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(500):
+            planner.run(idx, avail, n_sms)
+        torch.cuda.synchronize()
+        extras["planner_run_wall_us"] = round((time.perf_counter() - t) / 500 * 1e6, 2)
+
+    # ------------------------------------------------------------ CPU baseline
+    torch.set_num_threads(1)
+    idx_h, counts_h = inp.indices, inp.global_counts
+
+    def cpu_plan():
+        by = oracle.count_idx(idx_h, cfg.n_logical, n_sms)
+        o_res, _, _ = oracle.solve(counts_h, cfg.r2o, inp.phy2log, 1, C, n_fixed)
+        return oracle.map_idx(idx_h, o_res, by, o2r_host, inp.phy2log, 1, C, P)
+
+    cpu_plan()
+    cpu_us = []
+    t_end = time.perf_counter() + args.cpu_seconds
+    while time.perf_counter() < t_end:
+        t = time.perf_counter_ns()
+        cpu_plan()
+        cpu_us.append((time.perf_counter_ns() - t) / 1e3)
+    cpu_baseline = {"value": round(pct(cpu_us, 50), 1), "unit": "us per plan (p50)", "cores": 1, "kind": "port",
+                    "sample": f"{len(cpu_us)} plans of the same v3_ep8_cube inputs in {args.cpu_seconds:.0f} s, "
+                              f"scalar C restatement of the reference algorithm, host has {os.cpu_count()} CPUs",
+                    "p99": round(pct(cpu_us, 99), 1)}
+
+    line = {
+        "metric": "p50 us per plan (histogram + LP solve + redirect), EP8 cube V3 shape",
+        "value": round(p50, 2),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int64 indices, f32 LP with f64 normal-equation solve",
+        "data": "synthetic",
+        "config": {"workload": "v3_ep8_cube: 256 logical + 16 redundant experts, EP8 cube r2o, int64 indices "
+                               "[8192 x 8], global counts Zipf(1.0) x lognormal(0.3), n_blocks = CU count",
+                   "n_blocks": n_sms},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

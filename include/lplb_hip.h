@@ -44,6 +44,25 @@ int lplb_abi_version(void);
 const char *lplb_last_error(void);
 
 /*
+ * Profiling aid, no counterpart in the reference.  The next kernel this thread
+ * launches through the library records its own begin and end timestamps into
+ * the two hipEvent_t (either may be NULL); hipEventElapsedTime(start, stop)
+ * then gives that kernel's execution time, the figure a kernel trace reports,
+ * without the launch overhead an event pair around the call would include.
+ * The pair is consumed by that one launch.
+ */
+void lplb_time_next_launch(void *start_event, void *stop_event);
+
+/*
+ * Measurement aid, no counterpart in the reference: a plain streaming copy of
+ * n_elements int64 (even count) from src to dst.  Its achieved bandwidth is the
+ * practical ceiling the redirect kernel is compared with, and its known traffic
+ * (8 bytes read + 8 written per element) calibrates the profiler's byte counters.
+ */
+int lplb_copy_calibration(const int64_t *src, int64_t *dst, int64_t n_elements,
+                          lplb_stream_t stream);
+
+/*
  * Per-expert token histogram with an inclusive prefix over slices.
  * Replaces CompiledSolver.count_idx (csrc/plugin.cpp:580-600, kernel
  * minilp.cu:410-443).
@@ -129,6 +148,29 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
                  int group_size, int dup_per_rank, int n_combined_experts,
                  int n_local_experts, int n_blocks, int64_t *out,
                  lplb_stream_t stream);
+
+/*
+ * One batch's whole plan in a single call: lplb_count_idx, lplb_solve and
+ * lplb_map_idx chained on `stream`, i.e. what Planner.run does with three
+ * extension calls (lplb/planner.py:245-266).
+ *
+ *   global_counts    int32 [n_logical] or NULL.  NULL: the LP is fed this GPU's
+ *                    own histogram, as Planner.run does without a process
+ *                    group.  Otherwise the counts already summed over all EP
+ *                    ranks (what the all-reduce at lplb/planner.py:214-216
+ *                    yields).
+ *   counts_by_block  int32 [n_blocks, n_logical], out (see lplb_count_idx)
+ *   global_workload  fp32 [n_logical], out (see lplb_solve)
+ *   o_weight         fp32 [n_group, group_size, dup_per_rank], out
+ *   out              int64 [n_elements], out (see lplb_map_idx)
+ */
+int lplb_plan(const int64_t *idx, int64_t n_elements,
+              const int32_t *global_counts, const int32_t *r2o,
+              const int32_t *o2r, const int32_t *phy2log, int n_group,
+              int group_size, int dup_per_rank, int n_combined_experts,
+              int n_local_experts, int n_blocks, int32_t *counts_by_block,
+              float *global_workload, float *o_weight, int32_t *avail_num,
+              int64_t *out, int step_rule, int n_steps, lplb_stream_t stream);
 
 #ifdef __cplusplus
 }

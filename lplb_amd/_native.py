@@ -32,10 +32,13 @@ _i64 = ctypes.c_int64
 _SIGNATURES = {
     "lplb_abi_version": (_i, []),
     "lplb_last_error": (ctypes.c_char_p, []),
+    "lplb_time_next_launch": (None, [_vp, _vp]),
+    "lplb_copy_calibration": (_i, [_vp, _vp, _i64, _vp]),
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
 }
 
 
@@ -202,3 +205,48 @@ class CompiledSolver:
                                      self.dup_per_rank, self.n_combined_experts, self.n_local_experts, n_sms,
                                      out.data_ptr(), _stream(mapping_idx)))
         return out
+
+    # -- lplb/planner.py:245-266 in one library call -----------------------------
+    def plan(self, idx: torch.Tensor, r2o: torch.Tensor, o2r: torch.Tensor, phy2log: torch.Tensor,
+             avail_num: torch.Tensor, n_sms: int, global_counts: torch.Tensor | None = None,
+             workspace: dict | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Histogram, LP solve and redirect of one batch.  Returns (physical indices, o_weight,
+        counts per slice).  ``global_counts`` (int32 [n_logical]) replaces this GPU's own histogram
+        as the LP's workload.  ``workspace`` may carry preallocated ``out``, ``by_sm``, ``o_weight``
+        and ``global_workload`` tensors to reuse."""
+        _require(idx.dtype == torch.int64 and idx.is_cuda and idx.is_contiguous(),
+                 "idx is a contiguous int64 GPU tensor")
+        for name, t in (("r2o", r2o), ("o2r", o2r)):
+            _require(t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+                     and tuple(t.shape) == (self.group_size, self.dup_per_rank),
+                     f"{name} is a contiguous int32 [group_size, dup_per_rank] GPU tensor")
+        _require(phy2log.dtype == torch.int32 and phy2log.is_cuda and phy2log.is_contiguous()
+                 and phy2log.dim() == 1 and phy2log.size(0) == self.group_size * self.n_group * self.n_local_experts,
+                 "phy2log is a contiguous int32 [n_group * group_size * n_local_experts] GPU tensor")
+        _require(avail_num.numel() == 1 and avail_num.dtype == torch.int32 and avail_num.is_cuda,
+                 "avail_num is one int32 on the GPU")
+        if global_counts is not None:
+            _require(global_counts.dtype == torch.int32 and global_counts.is_cuda and global_counts.is_contiguous()
+                     and global_counts.numel() == self.n_experts, "global_counts is a contiguous int32 [n_experts] GPU tensor")
+        ws = workspace if workspace is not None else {}
+        dev = idx.device
+        out = ws.get("out")
+        if out is None or out.shape != idx.shape:
+            out = torch.empty_like(idx)
+        by_sm = ws.get("by_sm")
+        if by_sm is None or tuple(by_sm.shape) != (n_sms, self.n_experts):
+            by_sm = torch.empty((n_sms, self.n_experts), dtype=torch.int32, device=dev)
+        o_weight = ws.get("o_weight")
+        if o_weight is None:
+            o_weight = torch.empty((self.n_group, self.group_size, self.dup_per_rank), dtype=torch.float32, device=dev)
+        gw = ws.get("global_workload")
+        if gw is None:
+            gw = torch.empty(self.n_experts, dtype=torch.float32, device=dev)
+        _check(self.lib.lplb_plan(idx.data_ptr(), idx.numel(),
+                                  global_counts.data_ptr() if global_counts is not None else None,
+                                  r2o.data_ptr(), o2r.data_ptr(), phy2log.data_ptr(), self.n_group,
+                                  self.group_size, self.dup_per_rank, self.n_combined_experts,
+                                  self.n_local_experts, n_sms, by_sm.data_ptr(), gw.data_ptr(),
+                                  o_weight.data_ptr(), avail_num.data_ptr(), out.data_ptr(),
+                                  self.step_rule, self.n_steps, _stream(idx)))
+        return out, o_weight, by_sm

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/lplb_hip.h"
@@ -30,6 +31,24 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
       return ::lplb::fail(LPLB_EHIP, "%s failed: %s", #expr,                   \
                           hipGetErrorString(e_));                              \
   } while (0)
+
+// Events handed to lplb_time_next_launch() by this thread, cleared by the call.
+struct LaunchEvents {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+LaunchEvents take_launch_events();
+
+// Every kernel of the library is launched through here.  If the calling thread
+// armed a pair of events, the launch records the kernel's own begin and end
+// timestamps into them (not the time the launch was enqueued).
+template <typename Kernel, typename... Args>
+inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+  const LaunchEvents ev = take_launch_events();
+  if (ev.start || ev.stop)
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, ev.start, ev.stop, 0, args...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
+}
 
 // Length of one slice: ceil(n / parts) rounded up to kSliceAlign.
 __host__ __device__ inline int64_t slice_len(int64_t n, int parts) {

@@ -13,15 +13,20 @@
 
 namespace lplb {
 
-constexpr int kCountThreads = 256;
+constexpr int kLoadsInFlight = 4;   // 16-byte loads a thread issues before it consumes them
 
-__global__ __launch_bounds__(kCountThreads) void slice_histogram(
+__device__ inline void count_one(int32_t *hist, int64_t v, int n_experts) {
+  if (v >= 0 && v < n_experts)
+    atomicAdd(&hist[v], 1);
+}
+
+__global__ __launch_bounds__(1024) void slice_histogram(
     const int64_t *__restrict__ idx, int64_t n, int n_experts, int64_t per,
     int32_t *__restrict__ counts) {
   extern __shared__ int32_t hist[];
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, nt = blockDim.x;
   const int p = blockIdx.x;
-  for (int e = tid; e < n_experts; e += kCountThreads)
+  for (int e = tid; e < n_experts; e += nt)
     hist[e] = 0;
   __syncthreads();
 
@@ -30,49 +35,76 @@ __global__ __launch_bounds__(kCountThreads) void slice_histogram(
   // Slices start on multiples of 256 indices, so pairs are 16-byte aligned.
   const int64_t n_pairs = (end - begin) >> 1;
   const longlong2 *pairs = reinterpret_cast<const longlong2 *>(idx + begin);
-  for (int64_t i = tid; i < n_pairs; i += kCountThreads) {
-    longlong2 v = pairs[i];
-    if (v.x >= 0 && v.x < n_experts)
-      atomicAdd(&hist[v.x], 1);
-    if (v.y >= 0 && v.y < n_experts)
-      atomicAdd(&hist[v.y], 1);
+  for (int64_t i0 = tid; i0 < n_pairs; i0 += (int64_t)nt * kLoadsInFlight) {
+    longlong2 v[kLoadsInFlight];
+#pragma unroll
+    for (int u = 0; u < kLoadsInFlight; ++u) {
+      const int64_t i = i0 + (int64_t)u * nt;
+      v[u] = i < n_pairs ? pairs[i] : longlong2{-1, -1};
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsInFlight; ++u) {
+      count_one(hist, v[u].x, n_experts);
+      count_one(hist, v[u].y, n_experts);
+    }
   }
-  if (tid == 0 && ((end - begin) & 1)) {
-    int64_t v = idx[end - 1];
-    if (v >= 0 && v < n_experts)
-      atomicAdd(&hist[v], 1);
-  }
+  if (tid == 0 && ((end - begin) & 1))
+    count_one(hist, idx[end - 1], n_experts);
   __syncthreads();
   int32_t *row = counts + (int64_t)p * n_experts;
-  for (int e = tid; e < n_experts; e += kCountThreads)
+  for (int e = tid; e < n_experts; e += nt)
     row[e] = hist[e];
 }
 
 constexpr int kScanWaves = 16;
+constexpr int kScanRows = 16;   // rows a wave keeps in registers on the fast path
 
-// counts[p][e] <- sum_{p' <= p} counts[p'][e].
+// counts[p][e] <- sum_{p' <= p} counts[p'][e].  A workgroup owns 64 experts, its
+// waves own consecutive bands of rows; band sums meet in LDS.
 __global__ __launch_bounds__(kScanWaves *kWave) void prefix_over_slices(
     int32_t *__restrict__ counts, int n_blocks, int n_experts) {
   __shared__ int32_t part[kScanWaves][kWave];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int e = blockIdx.x * kWave + lane;
+  const bool live = e < n_experts;
   const int rows_per_wave = (n_blocks + kScanWaves - 1) / kScanWaves;
   const int r0 = min(n_blocks, wave * rows_per_wave);
   const int r1 = min(n_blocks, r0 + rows_per_wave);
+  int32_t *col = counts + e;
+  if (rows_per_wave <= kScanRows) {
+    // all loads in flight at once, scan in registers
+    int32_t v[kScanRows];
+#pragma unroll
+    for (int k = 0; k < kScanRows; ++k)
+      v[k] = (live && r0 + k < r1) ? col[(int64_t)(r0 + k) * n_experts] : 0;
+#pragma unroll
+    for (int k = 1; k < kScanRows; ++k)
+      v[k] += v[k - 1];
+    part[wave][lane] = v[kScanRows - 1];
+    __syncthreads();
+    int32_t offset = 0;
+    for (int w = 0; w < wave; ++w)
+      offset += part[w][lane];
+#pragma unroll
+    for (int k = 0; k < kScanRows; ++k)
+      if (live && r0 + k < r1)
+        col[(int64_t)(r0 + k) * n_experts] = v[k] + offset;
+    return;
+  }
   int32_t sum = 0;
-  if (e < n_experts)
+  if (live)
     for (int r = r0; r < r1; ++r)
-      sum += counts[(int64_t)r * n_experts + e];
+      sum += col[(int64_t)r * n_experts];
   part[wave][lane] = sum;
   __syncthreads();
   int32_t run = 0;
   for (int w = 0; w < wave; ++w)
     run += part[w][lane];
-  if (e < n_experts)
+  if (live)
     for (int r = r0; r < r1; ++r) {
-      run += counts[(int64_t)r * n_experts + e];
-      counts[(int64_t)r * n_experts + e] = run;
+      run += col[(int64_t)r * n_experts];
+      col[(int64_t)r * n_experts] = run;
     }
 }
 
@@ -91,14 +123,17 @@ extern "C" int lplb_count_idx(const int64_t *idx, int64_t n_elements,
   LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL,
                "count_idx: idx must be 16-byte aligned");
   const size_t lds = sizeof(int32_t) * (size_t)n_experts;
-  LPLB_REQUIRE(lds <= 160 * 1024, LPLB_EUNSUPPORTED,
+  LPLB_REQUIRE(lds <= 64 * 1024, LPLB_EUNSUPPORTED,
                "count_idx: n_experts=%d does not fit the LDS histogram", n_experts);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t per = slice_len(n_elements, n_blocks);
-  hipLaunchKernelGGL(slice_histogram, dim3(n_blocks), dim3(kCountThreads), lds, s, idx,
+  // one 16-byte load per thread covers 2 indices: 256 threads for slices of up to
+  // 2048 indices (4 loads each), 1024 threads beyond that
+  const int threads = per <= 2 * 256 * kLoadsInFlight ? 256 : 1024;
+  launch(slice_histogram, dim3(n_blocks), dim3(threads), lds, s, idx,
                      n_elements, n_experts, per, counts_by_block);
   LPLB_HIP_TRY(hipGetLastError());
-  hipLaunchKernelGGL(prefix_over_slices, dim3((n_experts + kWave - 1) / kWave),
+  launch(prefix_over_slices, dim3((n_experts + kWave - 1) / kWave),
                      dim3(kScanWaves * kWave), 0, s, counts_by_block, n_blocks, n_experts);
   LPLB_HIP_TRY(hipGetLastError());
   return LPLB_OK;

@@ -4,15 +4,18 @@
 // Each token needs its ordinal k among the tokens of the same expert, in index
 // order, because the original/replica decision hashes k.  The reference takes k
 // from a shared-memory atomic (minilp.cu:504), which fixes the set of ordinals
-// per block but not which token gets which.  Here k is canonical:
-//   * the slice of a workgroup is cut into contiguous sub-slices, one per wave;
-//   * phase A histograms every sub-slice into the wave's own LDS counter row;
-//   * phase B turns the rows into exclusive starting ordinals
-//     (previous slices' prefix + earlier waves of this slice);
-//   * phase C walks the sub-slice 64 indices at a time; lanes holding the same
-//     expert find each other with one ballot per expert-id bit, their rank among
-//     those peers is a popcount of lower lanes, and the last peer advances the
-//     wave's counter.  No atomics and two workgroup barriers in total.
+// per block but not which token gets which.  Here k is canonical.  A workgroup
+// walks its slice in rounds of n_waves * K * 64 indices; in a round every wave
+// owns K consecutive 64-index chunks, loaded once into registers with all loads
+// in flight together:
+//   A  each wave histograms its chunks into its own LDS counter row;
+//   B  the rows become exclusive starting ordinals (running total of earlier
+//      slices and rounds + earlier waves of this round);
+//   C  chunk by chunk, lanes holding the same expert find each other through a
+//      per-wave 64-bit LDS bitmap (one OR, one read); the rank among those peers
+//      is a popcount of lower lanes and the last peer advances the counter.
+// Two workgroup barriers per round, nothing order-dependent.  The modulo of the
+// hash uses a per-expert reciprocal prepared with the tables.
 #include "common.h"
 
 namespace lplb {
@@ -25,117 +28,171 @@ struct MapArgs {
   const int32_t *phy2log;
   int64_t n;
   int64_t per;
-  int n_logical, n_ranks, G, D, C, L, P, n_blocks, id_bits;
+  int n_logical, n_ranks, G, D, C, L, P, n_blocks;
   int64_t *out;
 };
 
-// Mask of the lanes whose (valid) key equals this lane's key.
-__device__ inline uint64_t match_any(int key, bool valid, int bits) {
-  uint64_t peers = __ballot(valid);
-  for (int b = 0; b < bits; ++b) {
-    const bool bit = (key >> b) & 1;
-    const uint64_t m = __ballot(bit);
-    peers &= bit ? m : ~m;
-  }
-  return peers;
+// Per-expert constants of the redirect, one 16-byte LDS read per token.
+struct __attribute__((aligned(16))) ExpertEntry {
+  int32_t total;     // tokens of this expert in the whole index array
+  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1)
+  int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
+  int32_t original;  // physical slot of the original
+};
+
+// |h| mod t with q = mulhi(|h|, magic): q is the true quotient or one less.
+__device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
+  if (x.total <= 0)
+    return 0;
+  const uint32_t a = h < 0 ? 0u - (uint32_t)h : (uint32_t)h;
+  uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
+  r = r >= (uint32_t)x.total ? r - (uint32_t)x.total : r;
+  return h < 0 ? -(int32_t)r : (int32_t)r;   // C's truncating %
 }
 
-__global__ __launch_bounds__(1024) void redirect_indices(MapArgs a) {
-  extern __shared__ int32_t smem[];
+constexpr int kMaxWaves = 16;
+
+template <int K>
+__global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int nl = a.n_logical;
-  int32_t *total = smem;
-  int32_t *expected = total + nl;
-  int32_t *log2r = expected + nl;    // [nl][2]: original slot, replica slot
-  int32_t *base = log2r + 2 * nl;    // [n_waves][nl]
   const int tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid % kWave, wave = tid / kWave, n_waves = nt / kWave;
   const int pid = blockIdx.x;
+  ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);                 // [nl]
+  unsigned long long *bitmap = reinterpret_cast<unsigned long long *>(table + nl); // [n_waves][nl]
+  int32_t *replica = reinterpret_cast<int32_t *>(bitmap + (size_t)n_waves * nl);   // [nl]
+  int32_t *carry = replica + nl;                                                   // [nl]
+  int32_t *base = carry + nl;                                                      // [n_waves][nl]
   const int32_t *last = a.by_block + (int64_t)(a.n_blocks - 1) * nl;
   const int32_t *prev = pid ? a.by_block + (int64_t)(pid - 1) * nl : nullptr;
 
-  // Tables, minilp.cu:466-496.
+  const int64_t begin = slice_begin(a.n, a.per, pid);
+  const int64_t end = slice_begin(a.n, a.per, pid + 1);
+  const int64_t round_len = (int64_t)n_waves * K * kWave;
+  int32_t *mine = base + wave * nl;
+  unsigned long long *my_bits = bitmap + (size_t)wave * nl;
+  const unsigned long long my_bit = 1ull << lane;
+
+  // First round's indices: issued before anything else so that their latency
+  // overlaps the table build.  ev = expert id, or -1 for masked / out-of-range /
+  // past the end.
+  int32_t ev[K];
+  auto load_round = [&](int64_t round) {
+    const int64_t wbeg = round + (int64_t)wave * K * kWave;
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const int64_t i = wbeg + c * kWave + lane;
+      const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
+      ev[c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
+    }
+  };
+  load_round(begin);
+
+  // Tables, minilp.cu:466-496.  All global reads of the build are independent of
+  // each other; the replicas' totals come back from LDS after the barrier.
+  const int cd = a.C * a.D;
   for (int e = tid; e < nl; e += nt) {
-    total[e] = expected[e] = last[e];
-    log2r[2 * e] = -1;
-    log2r[2 * e + 1] = -1;
-    for (int w = 0; w < n_waves; ++w)
-      base[w * nl + e] = 0;
+    const int32_t t = last[e];
+    const int32_t start = prev ? prev[e] : 0;
+    table[e].total = t;
+    table[e].magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : 0xffffffffu;
+    table[e].expected = t;
+    table[e].original = -1;
+    replica[e] = -1;
+    carry[e] = start;
+  }
+  for (int i = tid; i < n_waves * nl; i += nt) {
+    base[i] = 0;
+    bitmap[i] = 0;
   }
   __syncthreads();
   for (int e = tid; e < nl; e += nt) {
     const int slot = (e / a.L) * a.P + (e % a.L);
     const int le = a.phy2log[slot];
     if (le >= 0 && le < nl)
-      log2r[2 * le] = slot;
+      table[le].original = slot;
   }
-  const int cd = a.C * a.D;
   for (int i = tid; i < a.n_ranks * cd; i += nt) {
     const int ep_rank = i / cd, local = i % cd, d = local % a.D;
     const int le = a.phy2log[ep_rank * a.P + local];
+    const float share = a.o_weight[ep_rank * a.D + d];
+    const int host = a.o2r[(ep_rank % a.G) * a.D + d];
     if (le >= 0 && le < nl) {
       // fp32 product truncated toward zero (saturating, NaN -> 0)
-      expected[le] = __float2int_rz(a.o_weight[ep_rank * a.D + d] * (float)last[le]);
-      const int group = ep_rank / a.G, group_rank = ep_rank % a.G;
-      log2r[2 * le + 1] = (group * a.G + a.o2r[group_rank * a.D + d] + 1) * a.P - cd + local;
+      table[le].expected = __float2int_rz(share * (float)table[le].total);
+      replica[le] = ((ep_rank / a.G) * a.G + host + 1) * a.P - cd + local;
     }
   }
+  // (the barrier of phase A below also publishes the tables)
 
-  // Sub-slice of this wave: whole 64-index chunks.
-  const int64_t begin = slice_begin(a.n, a.per, pid);
-  const int64_t end = slice_begin(a.n, a.per, pid + 1);
-  const int64_t chunks = (end - begin + kWave - 1) / kWave;
-  const int64_t chunks_per_wave = (chunks + n_waves - 1) / n_waves;
-  int64_t wbeg = begin + wave * chunks_per_wave * kWave;
-  if (wbeg > end)
-    wbeg = end;
-  int64_t wend = wbeg + chunks_per_wave * kWave;
-  if (wend > end)
-    wend = end;
-  int32_t *mine = base + wave * nl;
+  for (int64_t round = begin; round < end; round += round_len) {
+    const int64_t wbeg = round + (int64_t)wave * K * kWave;
+    if (round != begin) {
+      load_round(round);
+      // counter rows still hold the previous round's ordinals
+      __syncthreads();
+      for (int i = tid; i < n_waves * nl; i += nt)
+        base[i] = 0;
+      __syncthreads();
+    }
+    // Phase A.
+#pragma unroll
+    for (int c = 0; c < K; ++c)
+      if (ev[c] >= 0)
+        atomicAdd(&mine[ev[c]], 1);
+    __syncthreads();
+    // Phase B: all rows of an expert are read before any is rewritten.
+    for (int e = tid; e < nl; e += nt) {
+      int32_t cnt[kMaxWaves];
+#pragma unroll
+      for (int w = 0; w < kMaxWaves; ++w)
+        cnt[w] = w < n_waves ? base[w * nl + e] : 0;
+      int32_t run = carry[e];
+#pragma unroll
+      for (int w = 0; w < kMaxWaves; ++w)
+        if (w < n_waves) {
+          base[w * nl + e] = run;
+          run += cnt[w];
+        }
+      carry[e] = run;
+    }
+    __syncthreads();
+    // Phase C.
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const int e = ev[c];
+      const bool valid = e >= 0;
+      if (valid)
+        atomicOr(&my_bits[e], my_bit);
+      int64_t o = -1;
+      if (valid) {
+        const unsigned long long peers =
+            __hip_atomic_load(&my_bits[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        const int rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32),
+                                                   __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+        const int cnt = __popcll(peers);
+        const int32_t k = mine[e] + rank;
+        const ExpertEntry x = table[e];
+        // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
+        const int32_t h = hashed_mod((int32_t)((uint32_t)k * 499u + 41u), x);
+        o = h >= x.expected ? replica[e] : x.original;
+        if (rank == cnt - 1) {
+          mine[e] = k + 1;
+          my_bits[e] = 0;
+        }
+      }
+      const int64_t i = wbeg + c * kWave + lane;
+      if (i < end)
+        __builtin_nontemporal_store(o, a.out + i);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
 
-  // Phase A (base rows were zeroed before the first barrier).
-  for (int64_t i = wbeg + lane; i < wend; i += kWave) {
-    const int64_t v = a.idx[i];
-    if (v >= 0 && v < nl)
-      atomicAdd(&mine[v], 1);
-  }
-  __syncthreads();
-  // Phase B.
-  for (int e = tid; e < nl; e += nt) {
-    int32_t run = prev ? prev[e] : 0;
-    for (int w = 0; w < n_waves; ++w) {
-      const int32_t t = base[w * nl + e];
-      base[w * nl + e] = run;
-      run += t;
-    }
-  }
-  __syncthreads();
-  // Phase C.
-  for (int64_t pos = wbeg; pos < wend; pos += kWave) {
-    const int64_t i = pos + lane;
-    const bool in = i < wend;
-    const int64_t v = in ? a.idx[i] : -1;
-    const bool valid = v >= 0 && v < nl;
-    const int e = valid ? (int)v : 0;
-    const uint64_t peers = match_any(e, valid, a.id_bits);
-    int64_t o = -1;
-    if (valid) {
-      const int rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32),
-                                                 __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
-      const int cnt = __popcll(peers);
-      const int32_t k = mine[e] + rank;
-      // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
-      int32_t h = (int32_t)((uint32_t)k * 499u + 41u);
-      const int32_t t = total[e];
-      h = t > 0 ? h % t : 0;
-      o = log2r[2 * e + (h >= expected[e] ? 1 : 0)];
-      if (rank == cnt - 1)
-        mine[e] = k + 1;
-    }
-    if (in)
-      a.out[i] = o;
-    __builtin_amdgcn_wave_barrier();
-  }
+// LDS bytes for n_logical experts and w waves.
+static size_t map_lds_bytes(int n_logical, int w) {
+  return (size_t)n_logical * (sizeof(ExpertEntry) + 8 + (size_t)w * 12);
 }
 
 } // namespace lplb
@@ -168,21 +225,28 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   a.n_ranks = n_group * group_size; a.n_logical = a.n_ranks * L;
   a.G = group_size; a.D = dup_per_rank; a.C = n_combined_experts; a.L = L;
   a.P = n_local_experts; a.n_blocks = n_blocks; a.out = out;
-  a.id_bits = 0;
-  while ((1 << a.id_bits) < a.n_logical)
-    ++a.id_bits;
 
-  // One wave per 64-index chunk of the slice, up to 16 waves, as LDS allows.
-  int n_waves = (int)((a.per + kWave - 1) / kWave);
-  if (n_waves > 16)
-    n_waves = 16;
-  auto lds_bytes = [&](int w) { return sizeof(int32_t) * (size_t)a.n_logical * (4 + w); };
-  while (n_waves > 1 && lds_bytes(n_waves) > 64 * 1024)
+  // One wave per 64-index chunk of the slice, up to 16 waves, as LDS allows;
+  // then up to 8 chunks per wave and round.
+  const int64_t chunks = (a.per + kWave - 1) / kWave;
+  int n_waves = chunks < kMaxWaves ? (int)chunks : kMaxWaves;
+  constexpr size_t kLdsLimit = 64 * 1024;
+  while (n_waves > 1 && map_lds_bytes(a.n_logical, n_waves) > kLdsLimit)
     n_waves >>= 1;
-  LPLB_REQUIRE(lds_bytes(n_waves) <= 64 * 1024, LPLB_EUNSUPPORTED,
+  LPLB_REQUIRE(map_lds_bytes(a.n_logical, n_waves) <= kLdsLimit, LPLB_EUNSUPPORTED,
                "map_idx: %d logical experts do not fit the LDS tables", a.n_logical);
-  hipLaunchKernelGGL(redirect_indices, dim3(n_blocks), dim3(n_waves * kWave), lds_bytes(n_waves),
-                     static_cast<hipStream_t>(stream), a);
+  const int64_t per_wave = (chunks + n_waves - 1) / n_waves;
+  const size_t lds = map_lds_bytes(a.n_logical, n_waves);
+  const dim3 grid(n_blocks), block(n_waves * kWave);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (per_wave <= 1)
+    launch(redirect_indices<1>, grid, block, lds, s, a);
+  else if (per_wave <= 2)
+    launch(redirect_indices<2>, grid, block, lds, s, a);
+  else if (per_wave <= 4)
+    launch(redirect_indices<4>, grid, block, lds, s, a);
+  else
+    launch(redirect_indices<8>, grid, block, lds, s, a);
   LPLB_HIP_TRY(hipGetLastError());
   return LPLB_OK;
 }

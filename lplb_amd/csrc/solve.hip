@@ -41,7 +41,22 @@ struct SolveArgs {
   int32_t *avail;
   float *result;             // [n_inst][n_group][G][D]
   int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps;
+#ifdef LPLB_PHASE_CLOCKS
+  long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0
+#endif
 };
+
+// Debug builds (-DLPLB_PHASE_CLOCKS) record the 100 MHz wall clock at phase
+// boundaries of the first wave; product builds compile the stamps away.
+#ifdef LPLB_PHASE_CLOCKS
+#define LPLB_STAMP(k)                                                          \
+  do {                                                                         \
+    if (a.clocks && blockIdx.x == 0 && threadIdx.x == 0)                       \
+      a.clocks[k] = wall_clock64();                                            \
+  } while (0)
+#else
+#define LPLB_STAMP(k)
+#endif
 
 template <int CTRL> __device__ inline float dpp(float v) {
   return __builtin_bit_cast(
@@ -52,231 +67,290 @@ constexpr int kQuadSwap2 = 0x4E;    // quad_perm [2,3,0,1]
 constexpr int kHalfMirror = 0x141;  // reverse within 8 lanes
 constexpr int kRowMirror = 0x140;   // reverse within 16 lanes
 
-// Sum over the 64 lanes; every lane gets the same bits.
-__device__ inline float reduce_sum(float v) {
+// Sum of lanes [0, W) (W = 8, 16, 32 or 64; lanes beyond W may hold anything for
+// W < 64 as long as whole 16-lane rows are either inside or outside).  The result
+// is wave-uniform.
+template <int W> __device__ inline float reduce_sum(float v) {
   v += dpp<kQuadSwap1>(v);
   v += dpp<kQuadSwap2>(v);
   v += dpp<kHalfMirror>(v);
+  if (W <= 8)
+    return readlane(v, 0);
   v += dpp<kRowMirror>(v);
+  if (W <= 16)
+    return readlane(v, 0);
+  if (W <= 32)
+    return readlane(v, 0) + readlane(v, 16);
   return (readlane(v, 0) + readlane(v, 16)) + (readlane(v, 32) + readlane(v, 48));
 }
 // Max with fmaxf semantics (NaN ignored unless everything is NaN).
-__device__ inline float reduce_max(float v) {
+template <int W> __device__ inline float reduce_max(float v) {
   v = fmaxf(v, dpp<kQuadSwap1>(v));
   v = fmaxf(v, dpp<kQuadSwap2>(v));
   v = fmaxf(v, dpp<kHalfMirror>(v));
+  if (W <= 8)
+    return readlane(v, 0);
   v = fmaxf(v, dpp<kRowMirror>(v));
+  if (W <= 16)
+    return readlane(v, 0);
+  if (W <= 32)
+    return fmaxf(readlane(v, 0), readlane(v, 16));
   return fmaxf(fmaxf(readlane(v, 0), readlane(v, 16)), fmaxf(readlane(v, 32), readlane(v, 48)));
 }
 
-// 1/sqrt(a) in fp64: hardware estimate + two Newton steps.
-__device__ inline double rsqrt_f64(double a) {
-  double r = __builtin_amdgcn_rsq(a);
-  r = r * (1.5 - 0.5 * a * r * r);
-  r = r * (1.5 - 0.5 * a * r * r);
-  return r;
+// 1/a in fp64: hardware estimate (about 2^-23) + one Newton step.
+__device__ inline double rcp_f64(double a) {
+  double r = __builtin_amdgcn_rcp(a);
+  return __builtin_fma(__builtin_fma(-a, r, 1.0), r, r);
 }
 
-template <int GM, int DM>
+// GM, DM: register-array sizes (group size and replica slots rounded up).
+// EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
+// constant; otherwise rows and columns G..GM-1 of the normal-equation system are
+// padded with the identity, which keeps the factorisation free of branches.
+template <int GM, int DM, bool EXACT>
 __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
-  // GM and DM only size the register arrays; the host checks G*D <= 64 edges.
   constexpr int T = kWave / GM;      // lanes that share the work of one rank's b_i
-  constexpr int LS = GM + 1;         // padded row stride of the transpose buffer
+  constexpr int LS = kWave + 1;      // row stride of the transpose buffer (doubles)
+  constexpr int NE = 2 * DM;         // replica edges that touch one rank
+  constexpr int KB = 4;              // fixed-expert counts a lane prefetches for b_i
+  constexpr int WR = GM;             // lanes that can hold a rank
+  constexpr int WE = GM * DM < kWave ? (GM * DM < 8 ? 8 : GM * DM) : kWave;  // ... an edge
+  constexpr int KG = 4;              // normalised counts a lane prefetches for the output
   __shared__ double lt_buf[GM * LS];
+  __shared__ int rep_of_edge[kWave];
 
   const int lane = threadIdx.x;
-  const int G = a.G, D = a.D, C = a.C, n = G * D;
-  const int L = D * C + a.n_fixed, P = L + D * C;
+  const int G = EXACT ? GM : a.G, D = EXACT ? DM : a.D;
+  const int C = a.C, n = G * D, n_fixed = a.n_fixed;
+  const int L = D * C + n_fixed, P = L + D * C;
   const int grp = blockIdx.x % a.n_group, inst = blockIdx.x / a.n_group;
-  const int32_t *wl = a.workload + (int64_t)inst * a.n_experts;
-  const int32_t *p2l = a.phy2log + (int64_t)grp * G * P;
-
-  // Normalisation by the maximum over all experts of all groups (minilp.cu:181-189).
-  float wmax = 0.0f;
-  for (int i = lane; i < a.n_experts; i += kWave)
-    wmax = fmaxf(wmax, (float)wl[i]);
-  wmax = reduce_max(wmax);
-  if (a.gw_out) {
-    float *gw = a.gw_out + (int64_t)inst * a.n_experts;
-    for (int i = grp * G * L + lane; i < (grp + 1) * G * L; i += kWave)
-      gw[i] = (float)wl[i] / wmax;
-  }
-  auto norm_count = [&](int e) -> float {
-    return (e >= 0 && e < a.n_experts) ? (float)wl[e] / wmax : 0.0f;
-  };
-
-  // ---- per-edge constants (lane j < n) ----
-  const bool is_edge = lane < n;
+  const int32_t *__restrict__ wl = a.workload + (int64_t)inst * a.n_experts;
+  const int32_t *__restrict__ p2l = a.phy2log + (int64_t)grp * G * P;
+  const bool is_edge = lane < n, is_rank = lane < G;
   const int ek = is_edge ? lane / D : 0;   // original rank of my edge
   const int ed = is_edge ? lane % D : 0;   // its replica slot
-  float w = 0.0f;                          // minilp.cu:203-221
-  if (is_edge)
-    for (int c = 0; c < C; ++c)
-      w += norm_count(p2l[ek * P + c * D + ed]);
-  int erep = ek;                           // rank holding the copy of my edge
-  if (is_edge)
-    for (int i = 0; i < G; ++i)
-      if (a.r2o[i * D + ed] == ek)
-        erep = i;
+  auto count_of = [&](int e) -> int { return (e >= 0 && e < a.n_experts) ? wl[e] : 0; };
 
+  LPLB_STAMP(0);
+  // ---- all global reads up front, as independent loads ----
+  // (a) the maximum over all experts of all groups, minilp.cu:181-189
+  float wmax = 0.0f;
+#pragma unroll 4
+  for (int i = lane; i < a.n_experts; i += kWave)
+    wmax = fmaxf(wmax, (float)wl[i]);
+  // (b) my edge's experts: raw count of the first, the rest in the loop below
+  const int e_first = (is_edge && C > 0) ? p2l[ek * P + ed] : -1;
+  // (c) the experts of "my" rank that cannot move (T lanes share a rank)
+  const int br = lane / T, bsub = lane % T;
+  int fixed_e[KB];
+#pragma unroll
+  for (int u = 0; u < KB; ++u) {
+    const int j = bsub + u * T;
+    fixed_e[u] = (br < G && j < n_fixed) ? p2l[br * P + D * C + j] : -1;
+  }
+  // (d) topology row of my rank
+  int r2o_row[DM];
+#pragma unroll
+  for (int d = 0; d < DM; ++d) {
+    int k = (is_rank && d < D) ? a.r2o[lane * D + d] : 0;
+    r2o_row[d] = k < 0 ? 0 : (k >= G ? G - 1 : k);
+  }
+  // (e) this group's counts, for the normalised-count output at the end
+  int out_cnt[KG];
+#pragma unroll
+  for (int u = 0; u < KG; ++u) {
+    const int i = lane + u * kWave;
+    out_cnt[u] = (a.gw_out && i < G * L) ? wl[grp * G * L + i] : 0;
+  }
+  const int w_first = count_of(e_first);
+  int fixed_cnt[KB];
+#pragma unroll
+  for (int u = 0; u < KB; ++u)
+    fixed_cnt[u] = count_of(fixed_e[u]);
+  wmax = reduce_max<kWave>(wmax);
+
+  LPLB_STAMP(1);
+  // ---- per-edge constants (lane j < n): w_j, minilp.cu:203-221 ----
+  float w = is_edge && C > 0 ? (float)w_first / wmax : 0.0f;
+  if (is_edge)
+    for (int c = 1; c < C; ++c)
+      w += (float)count_of(p2l[ek * P + c * D + ed]) / wmax;
+  // rank that holds the copy of each edge: invert r2o through LDS
+  rep_of_edge[lane] = ek;
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int d = 0; d < DM; ++d)
+    if (is_rank && d < D)
+      rep_of_edge[r2o_row[d] * D + d] = lane;
+  __builtin_amdgcn_wave_barrier();
+  const int erep = rep_of_edge[lane];
+
+  LPLB_STAMP(2);
   // ---- per-rank constants (lane i < G) ----
-  const bool is_rank = lane < G;
-  int src_o[DM], src_r[DM], oth_o[DM], oth_r[DM];
-  float w_o[DM], w_r[DM];
+  // Edge e < DM: my own edge (i, e), other end = where its copy lives.
+  // Edge DM + d: the edge copied into my slot d, other end = its original rank.
+  // An inactive edge points at myself, which makes all its terms vanish.
+  int src[NE], oth[NE];
+  float w_e[NE];
+  bool slot_on[DM];
 #pragma unroll
   for (int d = 0; d < DM; ++d) {
     const bool on = is_rank && d < D;
-    int k = on ? a.r2o[lane * D + d] : 0;
-    k = k < 0 ? 0 : (k >= G ? G - 1 : k);
-    src_o[d] = on ? lane * D + d : 0;      // my d-th own edge
-    src_r[d] = on ? k * D + d : 0;         // the edge whose copy sits in my slot d
-    oth_r[d] = k;
-    // Cross-lane reads stay outside any lane-dependent condition: a lane that
-    // is masked off would otherwise read as zero.
-    const int other = bpermute(erep, src_o[d]);
-    const float mine_w = bpermute(w, src_o[d]), copy_w = bpermute(w, src_r[d]);
-    oth_o[d] = on ? other : -1;
-    oth_r[d] = on ? k : -1;
-    w_o[d] = on ? mine_w : 0.0f;
-    w_r[d] = on ? copy_w : 0.0f;
+    slot_on[d] = on;
+    src[d] = on ? lane * D + d : 0;
+    src[DM + d] = on ? r2o_row[d] * D + d : 0;
+    // cross-lane reads stay outside lane-dependent conditions
+    const int other = bpermute(erep, src[d]);
+    const float w_own = bpermute(w, src[d]), w_copy = bpermute(w, src[DM + d]);
+    oth[d] = on ? other : lane;
+    oth[DM + d] = on ? r2o_row[d] : lane;
+    w_e[d] = on ? w_own : 0.0f;
+    w_e[DM + d] = on ? w_copy : 0.0f;
   }
-  // b_i = -(load of the experts that cannot move), minilp.cu:223-234; T lanes per rank.
+  // Selectors for assembling my row of S: 1 on my own column, -1 on the column
+  // of each edge's other end.
+  float mask[NE][GM], diag_mask[GM];
+#pragma unroll
+  for (int c = 0; c < GM; ++c) {
+    diag_mask[c] = (lane == c) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+      mask[e][c] = (oth[e] == c) ? -1.0f : 0.0f;
+  }
+
+  LPLB_STAMP(3);
+  // b_i = -(load of the experts that cannot move), minilp.cu:223-234
   float part = 0.0f;
-  {
-    const int r = lane / T, sub = lane % T;
-    if (r < G)
-      for (int j = sub; j < a.n_fixed; j += T)
-        part += norm_count(p2l[r * P + D * C + j]);
-    if (T >= 2) part += dpp<kQuadSwap1>(part);
-    if (T >= 4) part += dpp<kQuadSwap2>(part);
-    if (T >= 8) part += dpp<kHalfMirror>(part);
-  }
+#pragma unroll
+  for (int u = 0; u < KB; ++u)
+    part += (float)fixed_cnt[u] / wmax;
+  if (br < G)
+    for (int j = bsub + KB * T; j < n_fixed; j += T)
+      part += (float)count_of(p2l[br * P + D * C + j]) / wmax;
+  if (T >= 2) part += dpp<kQuadSwap1>(part);
+  if (T >= 4) part += dpp<kQuadSwap2>(part);
+  if (T >= 8) part += dpp<kHalfMirror>(part);
   const float part_of_rank = bpermute(part, (lane * T) & (kWave - 1));
   const float b = is_rank ? -part_of_rank : 0.0f;
   // Big-M column, minilp.cu:275-281: b_i minus the other entries of row i.
   float m = b;
 #pragma unroll
-  for (int d = 0; d < DM; ++d)
-    m -= w_o[d];
-#pragma unroll
-  for (int d = 0; d < DM; ++d)
-    m -= w_r[d];
+  for (int e = 0; e < NE; ++e)
+    m -= w_e[e];
   m = (m - 1.0f) + 1.0f;
   if (!is_rank)
     m = 0.0f;
 
+  LPLB_STAMP(4);
   // ---- affine scaling ----
   float xo = 1.0f, xr = 1.0f, xs = 1.0f, xt = 1.0f, xM = 1.0f;
   float d_max = 0.0f;
   const int NV = 2 * n + G + 2;
   const int win_lo = a.step_rule == LPLB_STEP_REFERENCE_WINDOW ? (NV > 32 ? NV - 32 : 0) : 0;
   const bool with_zero = a.step_rule != LPLB_STEP_REFERENCE_WINDOW || NV < 32;
+  const bool win_o = is_edge && lane >= win_lo, win_r = is_edge && n + lane >= win_lo;
+  const bool win_s = is_rank && 2 * n + lane >= win_lo;
+  const double row_on = is_rank ? 1.0 : 0.0;
 
   for (int step = 0; step < a.n_steps; ++step) {
     const float so = xo * xo, sr = xr * xr, ss = xs * xs, st = xt * xt, sM = xM * xM;
-    const float u = is_edge ? 1.0f / (so + sr) : 0.0f;
-    const float lam = w * w * so * sr * u;
-    const float ao = w * so * u, ar = w * sr * u;
-    const float sigma = reduce_sum(u);
-    const float kappa = sM / (1.0f + sM * sigma);
+    const float u = is_edge ? __builtin_amdgcn_rcpf(so + sr) : 0.0f;
+    const float wu = w * u;
+    const float ao = wu * so, ar = wu * sr;
+    const float lam = w * ao * sr;             // w^2 so sr / (so + sr)
+    const float sigma = reduce_sum<WE>(u);
+    const float kappa = sM * __builtin_amdgcn_rcpf(1.0f + sM * sigma);
 
-    float q = 0.0f;
-    double diag = (double)ss;
-    double lam_o[DM], lam_r[DM];
+    float q = 0.0f, lam_e[NE], lam_sum = ss;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float qo = bpermute(ao, src_o[d]), qr = bpermute(ar, src_r[d]);
-      const float lo = bpermute(lam, src_o[d]), lr = bpermute(lam, src_r[d]);
-      const bool on = oth_o[d] >= 0;
-      q += on ? qo + qr : 0.0f;
-      lam_o[d] = on ? (double)lo : 0.0;
-      lam_r[d] = on ? (double)lr : 0.0;
-      diag += lam_o[d] + lam_r[d];
+      const float q_own = bpermute(ao, src[d]), q_copy = bpermute(ar, src[DM + d]);
+      const float l_own = bpermute(lam, src[d]), l_copy = bpermute(lam, src[DM + d]);
+      // an inactive slot or a self-loop (oth == lane) contributes nothing to S;
+      // an inactive slot contributes nothing to q either
+      q += slot_on[d] ? q_own + q_copy : 0.0f;
+      lam_e[d] = (oth[d] == lane) ? 0.0f : l_own;
+      lam_e[DM + d] = (oth[DM + d] == lane) ? 0.0f : l_copy;
+      lam_sum += lam_e[d] + lam_e[DM + d];
     }
     const float v = is_rank ? m + q : 0.0f;
 
+    if (step == 0) LPLB_STAMP(5);
     // Row `lane` of S and its right-hand side, fp64.
     double S[GM];
-    const double dk = (double)kappa, dv = (double)v, dst = (double)st;
+    const double dst = (double)st, dkv = (double)kappa * (double)v;
+    const float st_col = is_rank ? st : 0.0f;
 #pragma unroll
     for (int c = 0; c < GM; ++c) {
-      double s = dst + dk * dv * (double)readlane(v, c);
+      float t = diag_mask[c] * lam_sum;
 #pragma unroll
-      for (int d = 0; d < DM; ++d) {
-        s -= (oth_o[d] == c) ? lam_o[d] : 0.0;
-        s -= (oth_r[d] == c) ? lam_r[d] : 0.0;
-      }
-      s += (lane == c) ? diag : 0.0;
-      S[c] = s;
+      for (int e = 0; e < NE; ++e)
+        t = __builtin_fmaf(mask[e][c], lam_e[e], t);
+      const double base = EXACT ? dst : (double)readlane(st_col, c) * row_on;
+      S[c] = __builtin_fma(dkv, (double)readlane(v, c), base) + (double)t;
     }
-    double rhs = 1000.0 * dk * dv - dst;
+    double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
 
-    // Cholesky S = L L^T with the forward substitution folded in.
-    double fwd = 0.0, my_rinv = 0.0;
+    if (step == 0) LPLB_STAMP(6);
+    // S = L D L^T by columns, forward substitution folded in.  The broadcast of
+    // column c to the trailing update reads un-normalised entries, so it does not
+    // wait for the pivot's reciprocal.
+    double my_pivot = 1.0;
 #pragma unroll
     for (int c = 0; c < GM; ++c) {
-      if (c < G) {
-        const double rinv = rsqrt_f64(readlane(S[c], c));
-        const double lc = S[c] * rinv;           // L[lane][c]
-        if (lane < GM)
-          lt_buf[c * LS + lane] = lc;
-        const double fc = readlane(rhs, c) * rinv;
-        if (lane == c) {
-          fwd = fc;
-          my_rinv = rinv;
-        }
-        rhs -= lc * fc;
+      const double pivot = readlane(S[c], c);
+      const double rinv = rcp_f64(pivot);
+      const double col = (lane > c) ? S[c] : 0.0;   // L[lane][c] * pivot
+      const double lc = col * rinv;                 // L[lane][c]
+      lt_buf[c * LS + lane] = lc;
+      my_pivot = (lane == c) ? pivot : my_pivot;
+      rhs = __builtin_fma(-lc, readlane(rhs, c), rhs);
 #pragma unroll
-        for (int c2 = c + 1; c2 < GM; ++c2)
-          if (c2 < G)
-            S[c2] -= lc * readlane(lc, c2);
-      }
+      for (int c2 = c + 1; c2 < GM; ++c2)
+        S[c2] = __builtin_fma(-lc, readlane(col, c2), S[c2]);
     }
+    if (step == 0) LPLB_STAMP(7);
     __builtin_amdgcn_wave_barrier();
-    // Lane c now takes column c of L.
+    // Lane c takes column c of L, then y = L^-T D^-1 z by a second column sweep.
     double LT[GM];
 #pragma unroll
     for (int i = 0; i < GM; ++i)
-      LT[i] = (lane < GM) ? lt_buf[lane * LS + i] : 0.0;
+      LT[i] = lane < GM ? lt_buf[lane * LS + i] : 0.0;
     __builtin_amdgcn_wave_barrier();
-    double acc = fwd, yd = 0.0;
+    // Entries L[i][c] with i <= c were stored as zeros, so step i leaves lanes
+    // >= i alone and lane i ends up holding y_i.
+    double acc = rhs * rcp_f64(my_pivot);
 #pragma unroll
-    for (int i = GM - 1; i >= 0; --i) {
-      if (i < G) {
-        const double yi = readlane(acc * my_rinv, i);
-        if (lane == i)
-          yd = yi;
-        acc -= LT[i] * yi;
-      }
-    }
-    const float y = is_rank ? (float)yd : 0.0f;
+    for (int i = GM - 1; i > 0; --i)
+      acc = __builtin_fma(-LT[i], readlane(acc, i), acc);
+    const float y = is_rank ? (float)acc : 0.0f;
 
+    if (step == 0) LPLB_STAMP(8);
     // r = A^T w and the direction d = x (c - r); the edge part of w is
     // z = u (h - kappa u.h + kappa (m.y - 1000)), h = -B^T y.
     const float yk = bpermute(y, ek), yrep = bpermute(y, erep);
     const float hp = -w * (so * yk + sr * yrep);
-    const float my = reduce_sum(m * y);
-    const float sumy = reduce_sum(y);
-    const float uh = reduce_sum(u * hp);
-    const float z = u * (hp - kappa * uh + kappa * (my - 1000.0f));
-    const float sumz = reduce_sum(z);
+    const float my = reduce_sum<WR>(m * y);
+    const float sumy = reduce_sum<WR>(y);
+    const float uh = reduce_sum<WE>(u * hp);
+    const float shift = kappa * (my - 1000.0f) - kappa * uh;
+    const float z = u * (hp + shift);
+    const float sumz = uh + shift * sigma;       // = sum of z over the edges
     const float d_o = -xo * (w * yk + z);
     const float d_r = -xr * (w * yrep + z);
     const float d_s = -xs * y;
     const float d_t = xt * (1.0f + sumy);
     const float d_M = xM * (1000.0f - (my - sumz));
 
+    if (step == 0) LPLB_STAMP(9);
     // Step length, minilp.cu:354-362.  NaN marks "not in the window".
     float cand = __builtin_nanf("");
-    if (is_edge && lane >= win_lo)
-      cand = fmaxf(cand, d_o);
-    if (is_edge && n + lane >= win_lo)
-      cand = fmaxf(cand, d_r);
-    if (is_rank && 2 * n + lane >= win_lo)
-      cand = fmaxf(cand, d_s);
-    if (lane == 0)
-      cand = fmaxf(fmaxf(cand, d_t), d_M);
-    d_max = reduce_max(cand);
+    cand = win_o ? fmaxf(cand, d_o) : cand;
+    cand = win_r ? fmaxf(cand, d_r) : cand;
+    cand = win_s ? fmaxf(cand, d_s) : cand;
+    cand = lane == 0 ? fmaxf(fmaxf(cand, d_t), d_M) : cand;
+    d_max = reduce_max<WE>(cand);
     if (with_zero)
       d_max = fmaxf(d_max, 0.0f);
     const float alpha = (float)(0.999 / (double)d_max);
@@ -285,22 +359,24 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     xs *= 1.0f - alpha * d_s;
     xt *= 1.0f - alpha * d_t;
     xM *= 1.0f - alpha * d_M;
+    if (step == 0) LPLB_STAMP(10);
   }
 
+  LPLB_STAMP(11);
   // Feasibility, minilp.cu:369-385.
   float res = 0.0f;
   {
     float row = xs - xt + m * xM - b;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float a_o = bpermute(xo, src_o[d]), a_r = bpermute(xr, src_r[d]);
-      row += w_o[d] * a_o + w_r[d] * a_r;
+      const float a_o = bpermute(xo, src[d]), a_r = bpermute(xr, src[DM + d]);
+      row += w_e[d] * a_o + w_e[DM + d] * a_r;
     }
     if (is_rank)
       res = fmaxf(res, fabsf(row));
     if (is_edge)
       res = fmaxf(res, fabsf(xo + xr - xM - 1.0f));
-    res = reduce_max(res);
+    res = reduce_max<WE>(res);
   }
   const bool ok = (double)d_max < 0.1 && 0.0 <= (double)xM && (double)xM < 1e-4 &&
                   (double)res < 0.05;
@@ -308,17 +384,31 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     atomicAdd(a.avail, 1);
   if (is_edge)
     a.result[(int64_t)blockIdx.x * n + lane] = ok ? xo : 0.5f;
+  // Normalised counts of this group, for the caller.
+  if (a.gw_out) {
+    float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;
+#pragma unroll
+    for (int u = 0; u < KG; ++u)
+      if (lane + u * kWave < G * L)
+        gw[lane + u * kWave] = (float)out_cnt[u] / wmax;
+    for (int i = lane + KG * kWave; i < G * L; i += kWave)
+      gw[i] = (float)wl[grp * G * L + i] / wmax;
+  }
+  LPLB_STAMP(12);
 }
 
-template <int GM, int DM> static void launch(const SolveArgs &a, int n_waves, hipStream_t s) {
-  hipLaunchKernelGGL((solve_groups<GM, DM>), dim3(n_waves), dim3(kWave), 0, s, a);
+template <int GM, int DM> static void launch_solver(const SolveArgs &a, int n_waves, hipStream_t s) {
+  if (a.G == GM && a.D == DM)
+    launch(solve_groups<GM, DM, true>, dim3(n_waves), dim3(kWave), 0, s, a);
+  else
+    launch(solve_groups<GM, DM, false>, dim3(n_waves), dim3(kWave), 0, s, a);
 }
 
 static int dispatch(const SolveArgs &a, int n_waves, hipStream_t s) {
   const int G = a.G, D = a.D;
 #define LPLB_CASE(GM, DM)                                                      \
   if (G <= GM && D <= DM) {                                                    \
-    launch<GM, DM>(a, n_waves, s);                                             \
+    launch_solver<GM, DM>(a, n_waves, s);                                             \
     return LPLB_OK;                                                            \
   }
   LPLB_CASE(8, 1) LPLB_CASE(8, 2) LPLB_CASE(8, 4) LPLB_CASE(8, 8)
@@ -329,7 +419,18 @@ static int dispatch(const SolveArgs &a, int n_waves, hipStream_t s) {
   return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
 }
 
+#ifdef LPLB_PHASE_CLOCKS
+static long long *g_phase_clocks = nullptr;
+#endif
+
 } // namespace lplb
+
+#ifdef LPLB_PHASE_CLOCKS
+// Debug builds only: device buffer of at least 16 int64 that receives the stamps.
+extern "C" void lplb_debug_set_phase_clocks(long long *device_buffer) {
+  lplb::g_phase_clocks = device_buffer;
+}
+#endif
 
 extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_workloads,
                                   const int32_t *r2o, const int32_t *phy2log,
@@ -362,6 +463,9 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
   a.avail = avail_num; a.result = results; a.n_group = n_group; a.G = group_size;
   a.D = dup_per_rank; a.C = n_experts_per_var; a.n_fixed = n_experts_fixed;
   a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps;
+#ifdef LPLB_PHASE_CLOCKS
+  a.clocks = g_phase_clocks;
+#endif
   int rc = dispatch(a, n_instances * n_group, static_cast<hipStream_t>(stream));
   if (rc != LPLB_OK)
     return rc;
