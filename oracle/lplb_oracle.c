@@ -57,11 +57,13 @@
 #undef FABS
 #undef FSQRT
 
-/* minilp.cu:404-408 */
+/* minilp.cu:404-408.  The reference computes in int; 64-bit intermediates give
+ * the same values wherever that does not overflow and stay defined up to
+ * n = INT_MAX. */
 int lplb_oracle_split_and_align(int n, int par_rank, int par_size, int align) {
-  int per = (n + par_size - 1) / par_size;
+  long long per = ((long long)n + par_size - 1) / par_size;
   per = (per + align - 1) / align * align;
-  long long v = (long long)per * par_rank;
+  long long v = per * par_rank;
   return v < n ? (int)v : n;
 }
 
