@@ -99,6 +99,11 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline sample")
     ap.add_argument("--skip-extras", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the redirect and copy kernels at the sweep shape (for counter collection)")
+    ap.add_argument("--roofline-reps", type=int, default=20, help="passes over the rotating buffers")
+    ap.add_argument("--solver-only", action="store_true",
+                    help="only 50 single and 10 batched (2048) LP solves at the plan's shape (for counter collection)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the plan; a run with --gpus > 1 is not supported "
@@ -142,6 +147,24 @@ def main() -> None:
     plan()
     ws["global_workload"] = torch.empty(cfg.n_logical, dtype=torch.float32, device=dev)
     torch.cuda.synchronize()
+    if args.roofline_only:
+        args.steps, args.warmup, args.skip_extras, args.cpu_seconds = 1, 0, True, 0.0
+    if args.solver_only:
+        lib_ = solver.lib
+        wl_ = counts.view(1, G, L)
+        gw_ = torch.empty(1, G, L, dtype=torch.float32, device=dev)
+        res_ = torch.empty(2048, 1, G, D, dtype=torch.float32, device=dev)
+        sweep_ = to_dev(synth.sweep_counts(2048).reshape(2048, 1, G, L))
+        st_ = torch.cuda.current_stream().cuda_stream
+        for _ in range(50):
+            assert lib_.lplb_solve(wl_.data_ptr(), gw_.data_ptr(), r2o.data_ptr(), phy2log.data_ptr(), 1, G, D, C,
+                                   n_fixed, avail.data_ptr(), res_.data_ptr(), 0, 5, st_) == 0
+        for _ in range(10):
+            assert lib_.lplb_solve_batched(sweep_.data_ptr(), None, r2o.data_ptr(), phy2log.data_ptr(), 2048, 1, G, D,
+                                           C, n_fixed, avail.data_ptr(), res_.data_ptr(), 0, 5, st_) == 0
+        torch.cuda.synchronize()
+        print(json.dumps({"solver_only": True, "feasible": int(avail[0])}))
+        return
 
     # ----------------------------------------------------------- timed region
     for _ in range(args.warmup):
@@ -184,7 +207,7 @@ def main() -> None:
                               sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_sms, bufs_out[i].data_ptr(), stream)
         assert rc == 0
 
-    reps = 20
+    reps = args.roofline_reps
     for i in range(n_buf):
         redirect(i)
     timer = KernelTimer(lib, reps * n_buf)
@@ -283,8 +306,10 @@ def main() -> None:
         o_res, _, _ = oracle.solve(counts_h, cfg.r2o, inp.phy2log, 1, C, n_fixed)
         return oracle.map_idx(idx_h, o_res, by, o2r_host, inp.phy2log, 1, C, P)
 
-    cpu_plan()
     cpu_us = []
+    t0c = time.perf_counter_ns()
+    cpu_plan()
+    cpu_us.append((time.perf_counter_ns() - t0c) / 1e3)
     t_end = time.perf_counter() + args.cpu_seconds
     while time.perf_counter() < t_end:
         t = time.perf_counter_ns()

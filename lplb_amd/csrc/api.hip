@@ -26,6 +26,10 @@ __global__ __launch_bounds__(1024) void copy_calibration(const i64x2 *__restrict
     __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+#ifdef LPLB_PHASE_CLOCKS
+long long *g_phase_clocks = nullptr;
+#endif
+
 static thread_local LaunchEvents g_launch_events;
 
 LaunchEvents take_launch_events() {
@@ -40,6 +44,13 @@ extern "C" void lplb_time_next_launch(void *start_event, void *stop_event) {
   lplb::g_launch_events.start = static_cast<hipEvent_t>(start_event);
   lplb::g_launch_events.stop = static_cast<hipEvent_t>(stop_event);
 }
+
+#ifdef LPLB_PHASE_CLOCKS
+// Debug builds only: device buffer of int64 that receives the stamps.
+extern "C" void lplb_debug_set_phase_clocks(long long *device_buffer) {
+  lplb::g_phase_clocks = device_buffer;
+}
+#endif
 
 extern "C" const char *lplb_last_error(void) { return lplb::g_last_error; }
 

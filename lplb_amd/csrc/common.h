@@ -50,6 +50,20 @@ inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
 }
 
+#ifdef LPLB_PHASE_CLOCKS
+// Debug builds only (-DLPLB_PHASE_CLOCKS): device buffer that receives the 100 MHz
+// wall clock at phase boundaries of selected waves; set with
+// lplb_debug_set_phase_clocks().  Product builds compile the stamps away.
+extern long long *g_phase_clocks;
+#define LPLB_STAMP_AT(ptr, k)                                                  \
+  do {                                                                         \
+    if ((ptr) && threadIdx.x == 0)                                             \
+      (ptr)[k] = wall_clock64();                                               \
+  } while (0)
+#else
+#define LPLB_STAMP_AT(ptr, k) do { } while (0)
+#endif
+
 // Length of one slice: ceil(n / parts) rounded up to kSliceAlign.
 __host__ __device__ inline int64_t slice_len(int64_t n, int parts) {
   int64_t per = (n + parts - 1) / parts;

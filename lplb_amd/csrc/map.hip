@@ -4,18 +4,22 @@
 // Each token needs its ordinal k among the tokens of the same expert, in index
 // order, because the original/replica decision hashes k.  The reference takes k
 // from a shared-memory atomic (minilp.cu:504), which fixes the set of ordinals
-// per block but not which token gets which.  Here k is canonical.  A workgroup
-// walks its slice in rounds of n_waves * K * 64 indices; in a round every wave
-// owns K consecutive 64-index chunks, loaded once into registers with all loads
-// in flight together:
-//   A  each wave histograms its chunks into its own LDS counter row;
-//   B  the rows become exclusive starting ordinals (running total of earlier
-//      slices and rounds + earlier waves of this round);
+// per block but not which token gets which.  Here k is canonical.
+//
+// A workgroup walks its slice in passes of R rounds; a round covers n_waves * K
+// consecutive 64-index chunks, K per wave.  All R*K loads of a pass are issued
+// up front (after the small table loads), then the rounds are processed in
+// order, each waiting only for its own loads (the host currently always picks
+// R = 1, see lplb_map_idx):
+//   A  each wave histograms its K chunks into its own LDS counter row;
+//   B  each wave turns the rows into its starting ordinals (running total of
+//      earlier slices and rounds + counts of the waves before it);
 //   C  chunk by chunk, lanes holding the same expert find each other through a
-//      per-wave 64-bit LDS bitmap (one OR, one read); the rank among those peers
-//      is a popcount of lower lanes and the last peer advances the counter.
-// Two workgroup barriers per round, nothing order-dependent.  The modulo of the
-// hash uses a per-expert reciprocal prepared with the tables.
+//      per-wave 64-bit LDS bitmap (one OR, one 16-byte read); the rank among those
+//      peers is a popcount of lower lanes and the last peer advances the counter.
+// Counter rows and running totals are double-buffered by round parity, which
+// leaves one workgroup barrier per round.  Nothing depends on execution order.
+// The modulo of the hash uses a per-expert reciprocal prepared with the tables.
 #include "common.h"
 
 namespace lplb {
@@ -30,29 +34,40 @@ struct MapArgs {
   int64_t per;
   int n_logical, n_ranks, G, D, C, L, P, n_blocks;
   int64_t *out;
+  long long *clocks;   // debug builds: stamps of the first and the last workgroup (else null)
 };
+#define LPLB_MAP_STAMP(k)                                                                      \
+  LPLB_STAMP_AT(blockIdx.x == 0 ? a.clocks + 32 : (blockIdx.x == gridDim.x - 1 ? a.clocks + 48 : nullptr), k)
 
 // Per-expert constants of the redirect, one 16-byte LDS read per token.
 struct __attribute__((aligned(16))) ExpertEntry {
   int32_t total;     // tokens of this expert in the whole index array
-  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1)
+  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1, 0 for total <= 0)
   int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
   int32_t original;  // physical slot of the original
 };
 
-// |h| mod t with q = mulhi(|h|, magic): q is the true quotient or one less.
-__device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
-  if (x.total <= 0)
-    return 0;
-  const uint32_t a = h < 0 ? 0u - (uint32_t)h : (uint32_t)h;
+// State of one expert inside one wave, one 16-byte LDS read / write per token.
+struct __attribute__((aligned(16))) WaveSlot {
+  int32_t next;             // ordinal of the wave's next token of this expert
+  int32_t unused;
+  unsigned long long bits;  // lanes of the current chunk that hold this expert
+};
+
+// h mod total with C's truncating sign rule; q = mulhi(|h|, magic) is the true
+// quotient or one less.  WRAP: the hash 499 k + 41 may have wrapped to negative.
+template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
+  const uint32_t a = WRAP ? (uint32_t)max(h, -h) : (uint32_t)h;
   uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
-  r = r >= (uint32_t)x.total ? r - (uint32_t)x.total : r;
-  return h < 0 ? -(int32_t)r : (int32_t)r;   // C's truncating %
+  r = min(r, r - (uint32_t)x.total);           // one conditional subtract
+  int32_t m = (WRAP && h < 0) ? -(int32_t)r : (int32_t)r;
+  return x.total > 0 ? m : 0;
 }
 
 constexpr int kMaxWaves = 16;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-template <int K>
+template <int K, int R, bool WRAP>
 __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int nl = a.n_logical;
@@ -60,139 +75,187 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   const int lane = tid % kWave, wave = tid / kWave, n_waves = nt / kWave;
   const int pid = blockIdx.x;
   ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);                 // [nl]
-  unsigned long long *bitmap = reinterpret_cast<unsigned long long *>(table + nl); // [n_waves][nl]
-  int32_t *replica = reinterpret_cast<int32_t *>(bitmap + (size_t)n_waves * nl);   // [nl]
-  int32_t *carry = replica + nl;                                                   // [nl]
-  int32_t *base = carry + nl;                                                      // [n_waves][nl]
+  WaveSlot *slots = reinterpret_cast<WaveSlot *>(table + nl);                    // [n_waves][nl]
+  int32_t *replica = reinterpret_cast<int32_t *>(slots + (size_t)n_waves * nl);  // [nl]
+  int32_t *carry = replica + nl;                                                 // [2][nl]
+  int32_t *counts = carry + 2 * nl;                                              // [2][n_waves][nl]
   const int32_t *last = a.by_block + (int64_t)(a.n_blocks - 1) * nl;
   const int32_t *prev = pid ? a.by_block + (int64_t)(pid - 1) * nl : nullptr;
 
   const int64_t begin = slice_begin(a.n, a.per, pid);
   const int64_t end = slice_begin(a.n, a.per, pid + 1);
   const int64_t round_len = (int64_t)n_waves * K * kWave;
-  int32_t *mine = base + wave * nl;
-  unsigned long long *my_bits = bitmap + (size_t)wave * nl;
+  WaveSlot *mine = slots + (size_t)wave * nl;
   const unsigned long long my_bit = 1ull << lane;
+  LPLB_MAP_STAMP(0);
 
-  // First round's indices: issued before anything else so that their latency
-  // overlaps the table build.  ev = expert id, or -1 for masked / out-of-range /
-  // past the end.
-  int32_t ev[K];
-  auto load_round = [&](int64_t round) {
-    const int64_t wbeg = round + (int64_t)wave * K * kWave;
-#pragma unroll
-    for (int c = 0; c < K; ++c) {
-      const int64_t i = wbeg + c * kWave + lane;
-      const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
-      ev[c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
-    }
-  };
-  load_round(begin);
-
-  // Tables, minilp.cu:466-496.  All global reads of the build are independent of
-  // each other; the replicas' totals come back from LDS after the barrier.
+  // Global reads of the table build (small, mostly L2 hits) go out first, the
+  // first pass's indices right behind them, so that the build does not wait for
+  // the bulk data.  Tables, minilp.cu:466-496.
   const int cd = a.C * a.D;
-  for (int e = tid; e < nl; e += nt) {
-    const int32_t t = last[e];
-    const int32_t start = prev ? prev[e] : 0;
-    table[e].total = t;
-    table[e].magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : 0xffffffffu;
-    table[e].expected = t;
-    table[e].original = -1;
+  const int e0 = tid;                                   // first (usually only) expert of this thread
+  const int32_t t0 = e0 < nl ? last[e0] : 0;
+  const int32_t s0 = (e0 < nl && prev) ? prev[e0] : 0;
+  const int le0 = e0 < nl ? a.phy2log[(e0 / a.L) * a.P + (e0 % a.L)] : -1;
+  const bool rep0 = tid < a.n_ranks * cd;               // first replicated expert set of this thread
+  const int rank0 = rep0 ? tid / cd : 0, local0 = rep0 ? tid % cd : 0;
+  const int rle0 = rep0 ? a.phy2log[rank0 * a.P + local0] : -1;
+  const float share0 = rep0 ? a.o_weight[rank0 * a.D + local0 % a.D] : 0.0f;
+  const int host0 = rep0 ? a.o2r[(rank0 % a.G) * a.D + local0 % a.D] : 0;
+
+  // Expert ids of one pass: -1 for masked / out-of-range / past the end.
+  int32_t ev[R][K];
+  auto load_pass = [&](int64_t pass) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int c = 0; c < K; ++c) {
+        const int64_t i = pass + r * round_len + ((int64_t)wave * K + c) * kWave + lane;
+        const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
+        ev[r][c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
+      }
+  };
+  load_pass(begin);
+
+  auto init_entry = [&](int e, int32_t t, int32_t start) {
+    ExpertEntry x;
+    x.total = t;
+    x.magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : (t == 1 ? 0xffffffffu : 0u);
+    x.expected = t;
+    x.original = -1;
+    table[e] = x;
     replica[e] = -1;
     carry[e] = start;
-  }
+  };
+  if (e0 < nl)
+    init_entry(e0, t0, s0);
+  for (int e = tid + nt; e < nl; e += nt)
+    init_entry(e, last[e], prev ? prev[e] : 0);
   for (int i = tid; i < n_waves * nl; i += nt) {
-    base[i] = 0;
-    bitmap[i] = 0;
+    slots[i] = WaveSlot{0, 0, 0ull};
+    counts[i] = 0;
+    counts[n_waves * nl + i] = 0;
   }
   __syncthreads();
-  for (int e = tid; e < nl; e += nt) {
-    const int slot = (e / a.L) * a.P + (e % a.L);
-    const int le = a.phy2log[slot];
+  auto set_original = [&](int e, int le) {
     if (le >= 0 && le < nl)
-      table[le].original = slot;
-  }
-  for (int i = tid; i < a.n_ranks * cd; i += nt) {
-    const int ep_rank = i / cd, local = i % cd, d = local % a.D;
-    const int le = a.phy2log[ep_rank * a.P + local];
-    const float share = a.o_weight[ep_rank * a.D + d];
-    const int host = a.o2r[(ep_rank % a.G) * a.D + d];
+      table[le].original = (e / a.L) * a.P + (e % a.L);
+  };
+  auto set_replica = [&](int ep_rank, int local, int le, float share, int host) {
     if (le >= 0 && le < nl) {
       // fp32 product truncated toward zero (saturating, NaN -> 0)
       table[le].expected = __float2int_rz(share * (float)table[le].total);
       replica[le] = ((ep_rank / a.G) * a.G + host + 1) * a.P - cd + local;
     }
+  };
+  if (e0 < nl)
+    set_original(e0, le0);
+  for (int e = tid + nt; e < nl; e += nt)
+    set_original(e, a.phy2log[(e / a.L) * a.P + (e % a.L)]);
+  if (rep0)
+    set_replica(rank0, local0, rle0, share0, host0);
+  for (int i = tid + nt; i < a.n_ranks * cd; i += nt) {
+    const int ep_rank = i / cd, local = i % cd, d = local % a.D;
+    set_replica(ep_rank, local, a.phy2log[ep_rank * a.P + local], a.o_weight[ep_rank * a.D + d],
+                a.o2r[(ep_rank % a.G) * a.D + d]);
   }
-  // (the barrier of phase A below also publishes the tables)
+  // (the barrier after the first phase A also publishes the tables)
+  LPLB_MAP_STAMP(1);
 
-  for (int64_t round = begin; round < end; round += round_len) {
-    const int64_t wbeg = round + (int64_t)wave * K * kWave;
-    if (round != begin) {
-      load_round(round);
-      // counter rows still hold the previous round's ordinals
-      __syncthreads();
-      for (int i = tid; i < n_waves * nl; i += nt)
-        base[i] = 0;
-      __syncthreads();
-    }
-    // Phase A.
+  int parity = 0;   // which half of counts / carry the current round uses
+  for (int64_t pass = begin; pass < end; pass += R * round_len) {
+    if (pass != begin)
+      load_pass(pass);
 #pragma unroll
-    for (int c = 0; c < K; ++c)
-      if (ev[c] >= 0)
-        atomicAdd(&mine[ev[c]], 1);
-    __syncthreads();
-    // Phase B: all rows of an expert are read before any is rewritten.
-    for (int e = tid; e < nl; e += nt) {
-      int32_t cnt[kMaxWaves];
+    for (int r = 0; r < R; ++r) {
+      const int64_t round = pass + r * round_len;
+      if (round < end) {   // uniform over the workgroup
+        int32_t *my_counts = counts + ((size_t)parity * n_waves + wave) * nl;
+        // Phase A: tokens per expert in this wave's chunks.
 #pragma unroll
-      for (int w = 0; w < kMaxWaves; ++w)
-        cnt[w] = w < n_waves ? base[w * nl + e] : 0;
-      int32_t run = carry[e];
+        for (int c = 0; c < K; ++c)
+          if (ev[r][c] >= 0)
+            atomicAdd(&my_counts[ev[r][c]], 1);
+        if (r == 0) LPLB_MAP_STAMP(2);
+        __syncthreads();
+        if (r == 0) LPLB_MAP_STAMP(3);
+        // Phase B: every wave derives its own starting ordinals: the running total
+        // of earlier slices and rounds plus the counts of the waves before it.  The
+        // last wave writes the next round's running total into the other half, and
+        // every wave clears its row of the other half for the next round.
+        const int32_t *round_counts = counts + (size_t)parity * n_waves * nl;
+        int32_t *other_counts = counts + ((size_t)(parity ^ 1) * n_waves + wave) * nl;
+        for (int e = lane; e < nl; e += kWave) {
+          // all reads in flight before the first add
+          int32_t before[kMaxWaves];
 #pragma unroll
-      for (int w = 0; w < kMaxWaves; ++w)
-        if (w < n_waves) {
-          base[w * nl + e] = run;
-          run += cnt[w];
+          for (int w = 0; w < kMaxWaves; ++w)
+            before[w] = w < wave ? round_counts[(size_t)w * nl + e] : 0;
+          int32_t run = carry[parity * nl + e];
+          const int32_t own = my_counts[e];
+#pragma unroll
+          for (int w = 0; w < kMaxWaves; ++w)
+            run += before[w];
+          mine[e].next = run;
+          if (wave == n_waves - 1)
+            carry[(parity ^ 1) * nl + e] = run + own;
+          other_counts[e] = 0;
         }
-      carry[e] = run;
-    }
-    __syncthreads();
-    // Phase C.
+        __builtin_amdgcn_wave_barrier();
+        if (r == 0) LPLB_MAP_STAMP(4);
+        // Phase C.
 #pragma unroll
-    for (int c = 0; c < K; ++c) {
-      const int e = ev[c];
-      const bool valid = e >= 0;
-      if (valid)
-        atomicOr(&my_bits[e], my_bit);
-      int64_t o = -1;
-      if (valid) {
-        const unsigned long long peers =
-            __hip_atomic_load(&my_bits[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-        const int rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32),
-                                                   __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
-        const int cnt = __popcll(peers);
-        const int32_t k = mine[e] + rank;
-        const ExpertEntry x = table[e];
-        // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
-        const int32_t h = hashed_mod((int32_t)((uint32_t)k * 499u + 41u), x);
-        o = h >= x.expected ? replica[e] : x.original;
-        if (rank == cnt - 1) {
-          mine[e] = k + 1;
-          my_bits[e] = 0;
+        for (int c = 0; c < K; ++c) {
+          const int e = ev[r][c];
+          const bool valid = e >= 0;
+          if (valid)
+            atomicOr(&mine[e].bits, my_bit);
+          int64_t o = -1;
+          if (valid) {
+            const i32x4 sraw = *reinterpret_cast<const i32x4 *>(&mine[e]);
+            const i32x4 xraw = *reinterpret_cast<const i32x4 *>(&table[e]);
+            const uint32_t peers_lo = (uint32_t)sraw.z, peers_hi = (uint32_t)sraw.w;
+            const int rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+            const int cnt = __popc(peers_lo) + __popc(peers_hi);
+            const int32_t k = sraw.x + rank;
+            ExpertEntry x;
+            x.total = xraw.x; x.magic = (uint32_t)xraw.y; x.expected = xraw.z; x.original = xraw.w;
+            // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
+            const int32_t h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
+            o = h >= x.expected ? replica[e] : x.original;
+            if (rank == cnt - 1)   // last peer: advance the ordinal, clear the bitmap
+              *reinterpret_cast<i32x4 *>(&mine[e]) = i32x4{k + 1, 0, 0, 0};
+          }
+          const int64_t i = round + ((int64_t)wave * K + c) * kWave + lane;
+          if (i < end)
+            __builtin_nontemporal_store(o, a.out + i);
+          __builtin_amdgcn_wave_barrier();
         }
+        if (r == 0) LPLB_MAP_STAMP(5);
+        parity ^= 1;
       }
-      const int64_t i = wbeg + c * kWave + lane;
-      if (i < end)
-        __builtin_nontemporal_store(o, a.out + i);
-      __builtin_amdgcn_wave_barrier();
     }
   }
+  __builtin_amdgcn_s_waitcnt(0);
+  LPLB_MAP_STAMP(6);
 }
 
 // LDS bytes for n_logical experts and w waves.
 static size_t map_lds_bytes(int n_logical, int w) {
-  return (size_t)n_logical * (sizeof(ExpertEntry) + 8 + (size_t)w * 12);
+  return (size_t)n_logical * (sizeof(ExpertEntry) + 4 + 8 + (size_t)w * (sizeof(WaveSlot) + 8));
+}
+
+template <int K, int R, bool WRAP>
+static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  if (lds > 64 * 1024) {
+    // above the default limit the kernel has to be told once per process
+    static hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&redirect_indices<K, R, WRAP>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (raised != hipSuccess)
+      return raised;
+  }
+  launch(redirect_indices<K, R, WRAP>, grid, block, lds, s, a);
+  return hipGetLastError();
 }
 
 } // namespace lplb
@@ -225,12 +288,17 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   a.n_ranks = n_group * group_size; a.n_logical = a.n_ranks * L;
   a.G = group_size; a.D = dup_per_rank; a.C = n_combined_experts; a.L = L;
   a.P = n_local_experts; a.n_blocks = n_blocks; a.out = out;
+#ifdef LPLB_PHASE_CLOCKS
+  a.clocks = g_phase_clocks;
+#else
+  a.clocks = nullptr;
+#endif
 
   // One wave per 64-index chunk of the slice, up to 16 waves, as LDS allows;
   // then up to 8 chunks per wave and round.
   const int64_t chunks = (a.per + kWave - 1) / kWave;
   int n_waves = chunks < kMaxWaves ? (int)chunks : kMaxWaves;
-  constexpr size_t kLdsLimit = 64 * 1024;
+  constexpr size_t kLdsLimit = 160 * 1024;
   while (n_waves > 1 && map_lds_bytes(a.n_logical, n_waves) > kLdsLimit)
     n_waves >>= 1;
   LPLB_REQUIRE(map_lds_bytes(a.n_logical, n_waves) <= kLdsLimit, LPLB_EUNSUPPORTED,
@@ -239,14 +307,26 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   const size_t lds = map_lds_bytes(a.n_logical, n_waves);
   const dim3 grid(n_blocks), block(n_waves * kWave);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (per_wave <= 1)
-    launch(redirect_indices<1>, grid, block, lds, s, a);
-  else if (per_wave <= 2)
-    launch(redirect_indices<2>, grid, block, lds, s, a);
-  else if (per_wave <= 4)
-    launch(redirect_indices<4>, grid, block, lds, s, a);
-  else
-    launch(redirect_indices<8>, grid, block, lds, s, a);
-  LPLB_HIP_TRY(hipGetLastError());
+  // 499 k + 41 stays below 2^31 for every ordinal k < n_elements
+  const bool wrap = n_elements > (INT32_MAX - 41) / 499;
+  hipError_t err;
+#define LPLB_MAP_CASE(K, R)                                                                    \
+  err = wrap ? launch_redirect<K, R, true>(a, grid, block, lds, s)                             \
+             : launch_redirect<K, R, false>(a, grid, block, lds, s)
+  // K chunks per wave and round, R rounds per pass (K * R loads in flight per
+  // lane).  Measured at [262144 x 8] on MI355X: a round costs about 2.5 us of
+  // barrier skew and counter traffic, more than splitting a pass into rounds can
+  // hide, so a pass is one round of up to 8 chunks; longer slices loop over passes.
+  if (per_wave <= 1) {
+    LPLB_MAP_CASE(1, 1);
+  } else if (per_wave <= 2) {
+    LPLB_MAP_CASE(2, 1);
+  } else if (per_wave <= 4) {
+    LPLB_MAP_CASE(4, 1);
+  } else {
+    LPLB_MAP_CASE(8, 1);
+  }
+#undef LPLB_MAP_CASE
+  LPLB_HIP_TRY(err);
   return LPLB_OK;
 }

@@ -41,22 +41,11 @@ struct SolveArgs {
   int32_t *avail;
   float *result;             // [n_inst][n_group][G][D]
   int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps;
-#ifdef LPLB_PHASE_CLOCKS
-  long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0
-#endif
+  long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
 
-// Debug builds (-DLPLB_PHASE_CLOCKS) record the 100 MHz wall clock at phase
-// boundaries of the first wave; product builds compile the stamps away.
-#ifdef LPLB_PHASE_CLOCKS
-#define LPLB_STAMP(k)                                                          \
-  do {                                                                         \
-    if (a.clocks && blockIdx.x == 0 && threadIdx.x == 0)                       \
-      a.clocks[k] = wall_clock64();                                            \
-  } while (0)
-#else
-#define LPLB_STAMP(k)
-#endif
+// Stamps of the first wave (debug builds only).
+#define LPLB_STAMP(k) LPLB_STAMP_AT(blockIdx.x == 0 ? a.clocks : nullptr, k)
 
 template <int CTRL> __device__ inline float dpp(float v) {
   return __builtin_bit_cast(
@@ -419,18 +408,7 @@ static int dispatch(const SolveArgs &a, int n_waves, hipStream_t s) {
   return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
 }
 
-#ifdef LPLB_PHASE_CLOCKS
-static long long *g_phase_clocks = nullptr;
-#endif
-
 } // namespace lplb
-
-#ifdef LPLB_PHASE_CLOCKS
-// Debug builds only: device buffer of at least 16 int64 that receives the stamps.
-extern "C" void lplb_debug_set_phase_clocks(long long *device_buffer) {
-  lplb::g_phase_clocks = device_buffer;
-}
-#endif
 
 extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_workloads,
                                   const int32_t *r2o, const int32_t *phy2log,
@@ -465,6 +443,8 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
   a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps;
 #ifdef LPLB_PHASE_CLOCKS
   a.clocks = g_phase_clocks;
+#else
+  a.clocks = nullptr;
 #endif
   int rc = dispatch(a, n_instances * n_group, static_cast<hipStream_t>(stream));
   if (rc != LPLB_OK)
