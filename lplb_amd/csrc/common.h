@@ -42,13 +42,22 @@ LaunchEvents take_launch_events();
 // armed a pair of events, the launch records the kernel's own begin and end
 // timestamps into them (not the time the launch was enqueued).
 template <typename Kernel, typename... Args>
-inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+inline void launch_with_flags(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                              unsigned flags, Args... args) {
   const LaunchEvents ev = take_launch_events();
-  if (ev.start || ev.stop)
-    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, ev.start, ev.stop, 0, args...);
+  if (ev.start || ev.stop || flags)
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, ev.start, ev.stop, flags, args...);
   else
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
 }
+template <typename Kernel, typename... Args>
+inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+  launch_with_flags(kernel, grid, block, lds, stream, 0u, args...);
+}
+
+// count.hip: histogram + scan; any_order lets it overlap the kernel enqueued just before it.
+int enqueue_count(const int64_t *idx, int64_t n_elements, int n_experts, int n_blocks,
+                  int32_t *counts_by_block, hipStream_t s, bool any_order);
 
 #ifdef LPLB_PHASE_CLOCKS
 // Debug builds only (-DLPLB_PHASE_CLOCKS): device buffer that receives the 100 MHz
@@ -60,8 +69,10 @@ extern long long *g_phase_clocks;
     if ((ptr) && threadIdx.x == 0)                                             \
       (ptr)[k] = wall_clock64();                                               \
   } while (0)
+inline long long *debug_clocks() { return g_phase_clocks; }
 #else
 #define LPLB_STAMP_AT(ptr, k) do { } while (0)
+inline long long *debug_clocks() { return nullptr; }
 #endif
 
 // Length of one slice: ceil(n / parts) rounded up to kSliceAlign.

@@ -3,11 +3,13 @@
 // Two launches on the caller's stream:
 //   1. slice_histogram: one workgroup per slice, LDS histogram fed by coalesced
 //      16-byte index loads, row p of the output = counts of slice p;
-//   2. prefix_over_slices: turns the rows into running sums down the slice
-//      axis.  A workgroup owns 64 experts (one per lane) and splits the slice
-//      axis over its waves, so the scan costs two short passes instead of the
-//      serial walk over all slices the reference does after its grid barrier
+//   2. prefix_over_slices: turns the rows into running sums down the slice axis,
+//      16 experts per workgroup and 16 row bands per expert, instead of the serial
+//      walk over all slices the reference does after its grid barrier
 //      (minilp.cu:439-442).
+// (Doing the scan inside the first kernel, by the last workgroup to finish, was
+// measured and rejected: one CU sustains too few outstanding misses to pull the
+// 256 KB table, 20 us against 3 us for this kernel.)
 // HBM-bound: 8 bytes read per index; the [n_blocks, n_experts] table is small.
 #include "common.h"
 
@@ -56,56 +58,74 @@ __global__ __launch_bounds__(1024) void slice_histogram(
     row[e] = hist[e];
 }
 
-constexpr int kScanWaves = 16;
-constexpr int kScanRows = 16;   // rows a wave keeps in registers on the fast path
+constexpr int kScanBands = 16;      // bands of rows, one per group of kScanCols lanes
+constexpr int kScanRows = 16;       // rows of a band a thread keeps in registers
+constexpr int kScanCols = 16;       // experts per workgroup: many small workgroups pull the
+                                    // table through many CUs (one CU sustains few misses)
 
-// counts[p][e] <- sum_{p' <= p} counts[p'][e].  A workgroup owns 64 experts, its
-// waves own consecutive bands of rows; band sums meet in LDS.
-__global__ __launch_bounds__(kScanWaves *kWave) void prefix_over_slices(
+// counts[p][e] <- sum_{p' <= p} counts[p'][e].  A workgroup owns kScanCols experts;
+// thread = (band of rows, expert).  All loads of a band are in flight at once
+// (clamped addresses, masked values); band sums meet in LDS; tables with more than
+// 256 slices take several sweeps with a running carry.
+__global__ __launch_bounds__(kScanBands *kScanCols) void prefix_over_slices(
     int32_t *__restrict__ counts, int n_blocks, int n_experts) {
-  __shared__ int32_t part[kScanWaves][kWave];
-  const int lane = threadIdx.x % kWave;
-  const int wave = threadIdx.x / kWave;
-  const int e = blockIdx.x * kWave + lane;
+  __shared__ int32_t part[kScanBands][kScanCols];
+  __shared__ int32_t carry[kScanCols];
+  const int col = threadIdx.x % kScanCols, band = threadIdx.x / kScanCols;
+  const int e = blockIdx.x * kScanCols + col;
   const bool live = e < n_experts;
-  const int rows_per_wave = (n_blocks + kScanWaves - 1) / kScanWaves;
-  const int r0 = min(n_blocks, wave * rows_per_wave);
-  const int r1 = min(n_blocks, r0 + rows_per_wave);
-  int32_t *col = counts + e;
-  if (rows_per_wave <= kScanRows) {
-    // all loads in flight at once, scan in registers
+  int32_t *column = counts + (live ? e : 0);
+  if (band == 0)
+    carry[col] = 0;
+  __syncthreads();
+  for (int row0 = 0; row0 < n_blocks; row0 += kScanBands * kScanRows) {
+    const int r0 = row0 + band * kScanRows;
     int32_t v[kScanRows];
 #pragma unroll
     for (int k = 0; k < kScanRows; ++k)
-      v[k] = (live && r0 + k < r1) ? col[(int64_t)(r0 + k) * n_experts] : 0;
+      v[k] = column[(int64_t)min(r0 + k, n_blocks - 1) * n_experts];
+#pragma unroll
+    for (int k = 0; k < kScanRows; ++k)
+      v[k] = (live && r0 + k < n_blocks) ? v[k] : 0;
 #pragma unroll
     for (int k = 1; k < kScanRows; ++k)
       v[k] += v[k - 1];
-    part[wave][lane] = v[kScanRows - 1];
+    part[band][col] = v[kScanRows - 1];
     __syncthreads();
-    int32_t offset = 0;
-    for (int w = 0; w < wave; ++w)
-      offset += part[w][lane];
+    int32_t offset = carry[col];
+#pragma unroll
+    for (int b = 0; b < kScanBands; ++b)
+      offset += b < band ? part[b][col] : 0;
 #pragma unroll
     for (int k = 0; k < kScanRows; ++k)
-      if (live && r0 + k < r1)
-        col[(int64_t)(r0 + k) * n_experts] = v[k] + offset;
-    return;
+      if (live && r0 + k < n_blocks)
+        column[(int64_t)(r0 + k) * n_experts] = v[k] + offset;
+    __syncthreads();
+    if (band == kScanBands - 1)
+      carry[col] = offset + v[kScanRows - 1];
+    __syncthreads();
   }
-  int32_t sum = 0;
-  if (live)
-    for (int r = r0; r < r1; ++r)
-      sum += col[(int64_t)r * n_experts];
-  part[wave][lane] = sum;
-  __syncthreads();
-  int32_t run = 0;
-  for (int w = 0; w < wave; ++w)
-    run += part[w][lane];
-  if (live)
-    for (int r = r0; r < r1; ++r) {
-      run += col[(int64_t)r * n_experts];
-      col[(int64_t)r * n_experts] = run;
-    }
+}
+
+// Enqueues histogram and prefix.  any_order: the histogram launch does not wait for
+// the kernel enqueued just before it on the stream (it still starts after everything
+// that kernel waited for); the prefix launch is ordered after both.
+int enqueue_count(const int64_t *idx, int64_t n_elements, int n_experts, int n_blocks,
+                  int32_t *counts_by_block, hipStream_t s, bool any_order) {
+  const size_t lds = sizeof(int32_t) * (size_t)n_experts;
+  LPLB_REQUIRE(lds <= 64 * 1024, LPLB_EUNSUPPORTED,
+               "count_idx: n_experts=%d does not fit the LDS histogram", n_experts);
+  const int64_t per = slice_len(n_elements, n_blocks);
+  // one 16-byte load per thread covers 2 indices: 256 threads for slices of up to
+  // 2048 indices (4 loads each), 1024 threads beyond that
+  const int threads = per <= 2 * 256 * kLoadsInFlight ? 256 : 1024;
+  launch_with_flags(slice_histogram, dim3(n_blocks), dim3(threads), lds, s,
+                    any_order ? hipExtAnyOrderLaunch : 0u, idx, n_elements, n_experts, per, counts_by_block);
+  LPLB_HIP_TRY(hipGetLastError());
+  launch(prefix_over_slices, dim3((n_experts + kScanCols - 1) / kScanCols), dim3(kScanBands * kScanCols), 0, s,
+         counts_by_block, n_blocks, n_experts);
+  LPLB_HIP_TRY(hipGetLastError());
+  return LPLB_OK;
 }
 
 } // namespace lplb
@@ -122,19 +142,6 @@ extern "C" int lplb_count_idx(const int64_t *idx, int64_t n_elements,
                "count_idx: null pointer");
   LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL,
                "count_idx: idx must be 16-byte aligned");
-  const size_t lds = sizeof(int32_t) * (size_t)n_experts;
-  LPLB_REQUIRE(lds <= 64 * 1024, LPLB_EUNSUPPORTED,
-               "count_idx: n_experts=%d does not fit the LDS histogram", n_experts);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t per = slice_len(n_elements, n_blocks);
-  // one 16-byte load per thread covers 2 indices: 256 threads for slices of up to
-  // 2048 indices (4 loads each), 1024 threads beyond that
-  const int threads = per <= 2 * 256 * kLoadsInFlight ? 256 : 1024;
-  launch(slice_histogram, dim3(n_blocks), dim3(threads), lds, s, idx,
-                     n_elements, n_experts, per, counts_by_block);
-  LPLB_HIP_TRY(hipGetLastError());
-  launch(prefix_over_slices, dim3((n_experts + kWave - 1) / kWave),
-                     dim3(kScanWaves * kWave), 0, s, counts_by_block, n_blocks, n_experts);
-  LPLB_HIP_TRY(hipGetLastError());
-  return LPLB_OK;
+  return enqueue_count(idx, n_elements, n_experts, n_blocks, counts_by_block,
+                       static_cast<hipStream_t>(stream), /*any_order=*/false);
 }

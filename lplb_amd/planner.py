@@ -153,6 +153,10 @@ class Planner:
         """
         if n_sms is None:
             n_sms = torch.cuda.get_device_properties(idx.device).multi_processor_count
+        if self.ep_group is None:
+            # count_workload -> solve_probs -> weighted_select_target in one library call
+            out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms)
+            return out
         local_workload, local_workload_by_sm = self.count_workload(idx, n_sms)
         o_weight, _global_workload = self.solve_probs(local_workload, avail_counter)
         return self.weighted_select_target(idx, o_weight, local_workload_by_sm, n_sms)

@@ -265,3 +265,116 @@ def test_redirect_full_size_sweep(cuda):
                 continue
             keep = int(np.clip(np.trunc(np.float32(w[rank, slot % shape.D]) * np.float32(tot[e])), 0, tot[e]))
             assert phys[rank * shape.P + slot] == keep, (rank, slot)
+
+
+# ------------------------------------------------------- single-call plan, graphs
+def _plan_setup(cuda, cfg_name, mask=0.05):
+    inp = synth.make_inputs(cfg_name, mask_fraction=mask)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    solver = solver_for(shape)
+    t = dict(idx=dev(inp.indices, cuda), r2o=dev(shape.r2o, cuda), o2r=dev(shape.o2r, cuda),
+             phy2log=dev(inp.phy2log, cuda), counts=dev(inp.global_counts, cuda))
+    return inp, shape, solver, t
+
+
+@pytest.mark.parametrize("cfg", ["cpu_ref_ep8", "v3_ep8_cube", "ep32_torus"])
+@pytest.mark.parametrize("use_global", [True, False])
+def test_plan_entry_point_matches_three_calls(cuda, cfg, use_global):
+    """lplb_plan == count_idx + solve + map_idx, with the LP fed by the supplied global counts or by
+    this GPU's own histogram (lplb/planner.py:264-266)."""
+    inp, shape, solver, t = _plan_setup(cuda, cfg)
+    n_sms = 200
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    out, o_weight, by_sm = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, n_sms,
+                                       global_counts=t["counts"] if use_global else None)
+    torch.cuda.synchronize()
+    want_by_sm = oracle.count_idx(inp.indices, shape.n_logical, n_sms)
+    np.testing.assert_array_equal(by_sm.cpu().numpy(), want_by_sm)
+    workload = inp.global_counts if use_global else want_by_sm[-1]
+    avail2 = torch.zeros(1, dtype=torch.int32, device=cuda)
+    ref_w, _ = solver.solve(dev(workload.reshape(shape.n_group, shape.G, shape.L), cuda), t["r2o"], t["phy2log"], avail2)
+    assert torch.equal(o_weight, ref_w) and int(avail[0]) == int(avail2[0]) == shape.n_group
+    want = oracle.map_idx(inp.indices, o_weight.cpu().numpy(), want_by_sm, shape.o2r, inp.phy2log, shape.n_group,
+                          shape.C, shape.P)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
+def test_planner_run_equals_plan_with_local_counts(cuda):
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    c = inp.cfg
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    planner.phy2log = t["phy2log"]
+    a1 = torch.zeros(1, dtype=torch.int32, device=cuda)
+    a2 = torch.zeros(1, dtype=torch.int32, device=cuda)
+    got = planner.run(t["idx"], a1, 128)
+    want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], a2, 128)
+    assert torch.equal(got, want) and int(a1[0]) == int(a2[0]) == 1
+
+
+def test_plan_replays_from_a_hip_graph(cuda):
+    """Capture two plans into a graph; every replay, with eager work and synchronisation between
+    replays, must reproduce the eager result and advance the counter."""
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    eager, eager_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])
+    torch.cuda.synchronize()
+    ws = {"out": torch.empty_like(eager), "o_weight": torch.empty_like(eager_w),
+          "by_sm": torch.empty(256, shape.n_logical, dtype=torch.int32, device=cuda),
+          "global_workload": torch.empty(shape.n_logical, dtype=torch.float32, device=cuda)}
+
+    def plan():
+        solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"], workspace=ws)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    before = int(avail[0])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan()
+        plan()
+    for rep in range(4):
+        ws["out"].fill_(-5)
+        ws["o_weight"].zero_()
+        scratch = torch.randn(1 << 16, device=cuda).sum()      # unrelated eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ws["out"], eager) and torch.equal(ws["o_weight"], eager_w), rep
+        assert int(avail[0]) == before + 2 * (rep + 1)
+        del scratch
+
+
+def test_kernel_timestamp_hook(cuda):
+    import ctypes
+    inp, shape, solver, t = _plan_setup(cuda, "cpu_ref_ep8")
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
+    total, by_sm = solver.count_idx(t["idx"], 16)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    solver.lib.lplb_time_next_launch(a, b)
+    res, _ = solver.solve(total.view(1, shape.G, shape.L), t["r2o"], t["phy2log"], avail)
+    torch.cuda.synchronize()
+    ms = ctypes.c_float()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+    assert 0.0 < ms.value < 5.0 and int(avail[0]) == 1
+    # the pair is consumed by one launch: the next call runs untimed and still works
+    res2, _ = solver.solve(total.view(1, shape.G, shape.L), t["r2o"], t["phy2log"], avail)
+    assert torch.equal(res, res2)
+
+
+@pytest.mark.parametrize("n,n_experts,n_sms", [(100000, 64, 700), (300000, 20, 1000), (5000, 7, 300)])
+def test_count_idx_many_slices(cuda, n, n_experts, n_sms):
+    """More than 256 slices: the prefix kernel takes several sweeps with a running carry."""
+    rng = np.random.default_rng(n)
+    idx = rng.integers(-1, n_experts, size=n, dtype=np.int64)
+    solver = CompiledSolver(1, 1, 1, n_experts + 1, 1)
+    _, by_sm = solver.count_idx(dev(idx, cuda), n_sms)
+    np.testing.assert_array_equal(by_sm.cpu().numpy(), oracle.count_idx(idx, n_experts, n_sms))
