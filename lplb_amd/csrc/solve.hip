@@ -24,14 +24,15 @@
 //     E_j = x_o^2 + x_r^2, u_j = 1/E_j, lambda_j = w_j^2 x_o^2 x_r^2 u_j,
 //     kappa = x_M^2 / (1 + x_M^2 sum u), q = B u, v = m + q.
 // Lane i of the wave owns rank i and row i of S, lane j owns edge j.  S is
-// assembled, factorised (right-looking Cholesky, pivots broadcast with
-// v_readlane) and solved in fp64: it is tiny, and fp64 here removes the
-// 1e-4..1e-3 rounding scatter a 32-bit factorisation shows on nearly balanced
-// loads.  Everything else is fp32.  The factor is transposed through LDS once per
-// step so that the backward substitution is also a column sweep.
+// assembled and [S | rhs] reduced by Gauss-Jordan elimination (pivots and pivot-row
+// entries broadcast with v_readlane, every lane updating its own row) in fp64: the
+// system is tiny, and fp64 here removes the 1e-4..1e-3 rounding scatter a 32-bit
+// factorisation shows on nearly balanced loads.  Everything else is fp32.
 #include "common.h"
 
 namespace lplb {
+
+constexpr int kStagedExperts = 2048;   // counts kept in LDS (8 KB) for the gathers
 
 struct SolveArgs {
   const int32_t *workload;   // [n_inst][n_experts]
@@ -100,13 +101,12 @@ __device__ inline double rcp_f64(double a) {
 template <int GM, int DM, bool EXACT>
 __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   constexpr int T = kWave / GM;      // lanes that share the work of one rank's b_i
-  constexpr int LS = kWave + 1;      // row stride of the transpose buffer (doubles)
   constexpr int NE = 2 * DM;         // replica edges that touch one rank
   constexpr int KB = 4;              // fixed-expert counts a lane prefetches for b_i
   constexpr int WR = GM;             // lanes that can hold a rank
   constexpr int WE = GM * DM < kWave ? (GM * DM < 8 ? 8 : GM * DM) : kWave;  // ... an edge
   constexpr int KG = 4;              // normalised counts a lane prefetches for the output
-  __shared__ double lt_buf[GM * LS];
+  __shared__ float staged_counts[kStagedExperts];
   __shared__ int rep_of_edge[kWave];
 
   const int lane = threadIdx.x;
@@ -119,15 +119,26 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   const bool is_edge = lane < n, is_rank = lane < G;
   const int ek = is_edge ? lane / D : 0;   // original rank of my edge
   const int ed = is_edge ? lane % D : 0;   // its replica slot
-  auto count_of = [&](int e) -> int { return (e >= 0 && e < a.n_experts) ? wl[e] : 0; };
+  // Up to kStagedExperts counts are staged in LDS as floats, so that the gathers
+  // through phy2log do not need a second round trip to global memory.
+  const bool staged = a.n_experts <= kStagedExperts;
+  auto count_of = [&](int e) -> float {
+    if (e < 0 || e >= a.n_experts)
+      return 0.0f;
+    return staged ? staged_counts[e] : (float)wl[e];
+  };
 
   LPLB_STAMP(0);
   // ---- all global reads up front, as independent loads ----
   // (a) the maximum over all experts of all groups, minilp.cu:181-189
   float wmax = 0.0f;
 #pragma unroll 4
-  for (int i = lane; i < a.n_experts; i += kWave)
-    wmax = fmaxf(wmax, (float)wl[i]);
+  for (int i = lane; i < a.n_experts; i += kWave) {
+    const float cnt = (float)wl[i];
+    wmax = fmaxf(wmax, cnt);
+    if (staged)
+      staged_counts[i] = cnt;
+  }
   // (b) my edge's experts: raw count of the first, the rest in the loop below
   const int e_first = (is_edge && C > 0) ? p2l[ek * P + ed] : -1;
   // (c) the experts of "my" rank that cannot move (T lanes share a rank)
@@ -152,8 +163,9 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     const int i = lane + u * kWave;
     out_cnt[u] = (a.gw_out && i < G * L) ? wl[grp * G * L + i] : 0;
   }
-  const int w_first = count_of(e_first);
-  int fixed_cnt[KB];
+  __builtin_amdgcn_wave_barrier();   // staged counts are visible to the whole wave
+  const float w_first = count_of(e_first);
+  float fixed_cnt[KB];
 #pragma unroll
   for (int u = 0; u < KB; ++u)
     fixed_cnt[u] = count_of(fixed_e[u]);
@@ -161,10 +173,10 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
 
   LPLB_STAMP(1);
   // ---- per-edge constants (lane j < n): w_j, minilp.cu:203-221 ----
-  float w = is_edge && C > 0 ? (float)w_first / wmax : 0.0f;
+  float w = is_edge && C > 0 ? w_first / wmax : 0.0f;
   if (is_edge)
     for (int c = 1; c < C; ++c)
-      w += (float)count_of(p2l[ek * P + c * D + ed]) / wmax;
+      w += count_of(p2l[ek * P + c * D + ed]) / wmax;
   // rank that holds the copy of each edge: invert r2o through LDS
   rep_of_edge[lane] = ek;
   __builtin_amdgcn_wave_barrier();
@@ -213,10 +225,10 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   float part = 0.0f;
 #pragma unroll
   for (int u = 0; u < KB; ++u)
-    part += (float)fixed_cnt[u] / wmax;
+    part += fixed_cnt[u] / wmax;
   if (br < G)
     for (int j = bsub + KB * T; j < n_fixed; j += T)
-      part += (float)count_of(p2l[br * P + D * C + j]) / wmax;
+      part += count_of(p2l[br * P + D * C + j]) / wmax;
   if (T >= 2) part += dpp<kQuadSwap1>(part);
   if (T >= 4) part += dpp<kQuadSwap2>(part);
   if (T >= 8) part += dpp<kHalfMirror>(part);
@@ -282,38 +294,25 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
 
     if (step == 0) LPLB_STAMP(6);
-    // S = L D L^T by columns, forward substitution folded in.  The broadcast of
-    // column c to the trailing update reads un-normalised entries, so it does not
-    // wait for the pivot's reciprocal.
+    // Gauss-Jordan elimination of [S | rhs] by columns: lane i owns row i, column c
+    // is cleared in every other row at once, so no triangular solves (and no
+    // transposed factor) are needed afterwards.  Row c's entries are read from lane
+    // c before they are scaled, so those broadcasts do not wait for the pivot's
+    // reciprocal.  S is symmetric positive definite: no pivoting.
     double my_pivot = 1.0;
 #pragma unroll
     for (int c = 0; c < GM; ++c) {
       const double pivot = readlane(S[c], c);
       const double rinv = rcp_f64(pivot);
-      const double col = (lane > c) ? S[c] : 0.0;   // L[lane][c] * pivot
-      const double lc = col * rinv;                 // L[lane][c]
-      lt_buf[c * LS + lane] = lc;
       my_pivot = (lane == c) ? pivot : my_pivot;
-      rhs = __builtin_fma(-lc, readlane(rhs, c), rhs);
+      const double f = (lane != c) ? S[c] * rinv : 0.0;   // multiple of row c to subtract from my row
+      rhs = __builtin_fma(-f, readlane(rhs, c), rhs);
 #pragma unroll
       for (int c2 = c + 1; c2 < GM; ++c2)
-        S[c2] = __builtin_fma(-lc, readlane(col, c2), S[c2]);
+        S[c2] = __builtin_fma(-f, readlane(S[c2], c), S[c2]);
     }
     if (step == 0) LPLB_STAMP(7);
-    __builtin_amdgcn_wave_barrier();
-    // Lane c takes column c of L, then y = L^-T D^-1 z by a second column sweep.
-    double LT[GM];
-#pragma unroll
-    for (int i = 0; i < GM; ++i)
-      LT[i] = lane < GM ? lt_buf[lane * LS + i] : 0.0;
-    __builtin_amdgcn_wave_barrier();
-    // Entries L[i][c] with i <= c were stored as zeros, so step i leaves lanes
-    // >= i alone and lane i ends up holding y_i.
-    double acc = rhs * rcp_f64(my_pivot);
-#pragma unroll
-    for (int i = GM - 1; i > 0; --i)
-      acc = __builtin_fma(-LT[i], readlane(acc, i), acc);
-    const float y = is_rank ? (float)acc : 0.0f;
+    const float y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
 
     if (step == 0) LPLB_STAMP(8);
     // r = A^T w and the direction d = x (c - r); the edge part of w is
