@@ -30,6 +30,10 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 REDIRECT_BYTES_PER_INDEX = 16
+# HBM bytes one redirect launch moves at the sweep shape, from rocprofv3 FETCH_SIZE and WRITE_SIZE (two
+# runs), each scaled by what the same counter reads for the plain copy kernel of known size:
+# 16 797 KiB read + 16 376 KiB written, 1.012 x the algorithmic bytes.
+REDIRECT_TRAFFIC_BYTES_SWEEP = 33_969_000
 HISTOGRAM_BYTES_PER_INDEX = 8
 
 
@@ -237,7 +241,7 @@ def main() -> None:
     copy_us = timer.times_us(torch)
     copy_gbs = alg_bytes / (float(copy_us.mean()) * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": REDIRECT_TRAFFIC_BYTES_SWEEP,
                 "kernel": "redirect_indices", "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64",
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
                 "p50_launch_us": round(pct(red_us, 50), 2), "distinct_buffer_pairs": n_buf,
