@@ -29,10 +29,11 @@
 // system is tiny, and fp64 here removes the 1e-4..1e-3 rounding scatter a 32-bit
 // factorisation shows on nearly balanced loads.  Everything else is fp32.
 #include "common.h"
+#include <type_traits>
+#include <utility>
 
 namespace lplb {
 
-constexpr int kStagedExperts = 2048;   // counts kept in LDS (8 KB) for the gathers
 
 struct SolveArgs {
   const int32_t *workload;   // [n_inst][n_experts]
@@ -41,7 +42,7 @@ struct SolveArgs {
   const int32_t *phy2log;    // [n_group][G][P]
   int32_t *avail;
   float *result;             // [n_inst][n_group][G][D]
-  int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps;
+  int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps, n_units;
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
 
@@ -94,34 +95,107 @@ __device__ inline double rcp_f64(double a) {
   return __builtin_fma(__builtin_fma(-a, r, 1.0), r, r);
 }
 
+// Calls f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>):
+// a loop whose index is a constant expression, as the DPP controls need.
+template <typename F, int... I> __device__ inline void static_for_impl(F &f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ inline void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// ---- one LP per wave (ROWS == 1) or one LP per 16-lane DPP row (ROWS == 4) ----
+// With ROWS == 4 a lane's position inside its row plays the part of the lane id,
+// broadcasts are row-local DPP moves (row_newbcast) and reductions stop at the
+// row, so four independent LPs share the wave's instruction stream.
+constexpr int kRowLanes = 16;
+template <int ROWS> struct Layout {
+  static constexpr int kWidth = ROWS == 1 ? kWave : kRowLanes;   // lanes that serve one LP
+};
+
+template <int LANE> __device__ inline float row_bcast(float v) { return dpp<0x150 + LANE>(v); }
+template <int LANE> __device__ inline double row_bcast(double v) {
+  int2 p = __builtin_bit_cast(int2, v);
+  p.x = __builtin_amdgcn_update_dpp(0, p.x, 0x150 + LANE, 0xF, 0xF, false);
+  p.y = __builtin_amdgcn_update_dpp(0, p.y, 0x150 + LANE, 0xF, 0xF, false);
+  return __builtin_bit_cast(double, p);
+}
+// Value of `v` in lane LANE of this LP's lanes.
+template <int ROWS, int LANE, typename T> __device__ inline T lp_bcast(T v) {
+  if constexpr (ROWS == 1)
+    return readlane(v, LANE);
+  else
+    return row_bcast<LANE>(v);
+}
+// Reductions over the first W lanes of this LP (W <= 16 when ROWS == 4).
+template <int ROWS, int W> __device__ inline float lp_sum(float v) {
+  if constexpr (ROWS == 1) {
+    return reduce_sum<W>(v);
+  } else {
+    v += dpp<kQuadSwap1>(v);
+    v += dpp<kQuadSwap2>(v);
+    v += dpp<kHalfMirror>(v);
+    if (W > 8)
+      v += dpp<kRowMirror>(v);
+    return row_bcast<0>(v);
+  }
+}
+template <int ROWS, int W> __device__ inline float lp_max(float v) {
+  if constexpr (ROWS == 1) {
+    return reduce_max<W>(v);
+  } else {
+    v = fmaxf(v, dpp<kQuadSwap1>(v));
+    v = fmaxf(v, dpp<kQuadSwap2>(v));
+    v = fmaxf(v, dpp<kHalfMirror>(v));
+    if (W > 8)
+      v = fmaxf(v, dpp<kRowMirror>(v));
+    return row_bcast<0>(v);
+  }
+}
+
 // GM, DM: register-array sizes (group size and replica slots rounded up).
 // EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
 // constant; otherwise rows and columns G..GM-1 of the normal-equation system are
 // padded with the identity, which keeps the factorisation free of branches.
-template <int GM, int DM, bool EXACT>
-__global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
-  constexpr int T = kWave / GM;      // lanes that share the work of one rank's b_i
+// ROWS: LPs per wave (1, or 4 when GM <= 16 and GM * DM <= 16).  WAVES: waves per
+// workgroup; they share nothing and never synchronise, a bigger workgroup only
+// means fewer of them to dispatch.
+template <int GM, int DM, bool EXACT, int ROWS, int WAVES>
+__global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
+  constexpr int WL = Layout<ROWS>::kWidth;   // lanes of one LP
+  static_assert(ROWS == 1 || (ROWS == 4 && GM <= kRowLanes && GM * DM <= kRowLanes), "an LP must fit its lanes");
+  constexpr int T = WL / GM;         // lanes that share the work of one rank's b_i
   constexpr int NE = 2 * DM;         // replica edges that touch one rank
-  constexpr int KB = 4;              // fixed-expert counts a lane prefetches for b_i
+  constexpr int KB = ROWS == 1 ? 4 : 16;   // fixed-expert counts a lane prefetches for b_i
   constexpr int WR = GM;             // lanes that can hold a rank
-  constexpr int WE = GM * DM < kWave ? (GM * DM < 8 ? 8 : GM * DM) : kWave;  // ... an edge
-  constexpr int KG = 4;              // normalised counts a lane prefetches for the output
-  __shared__ float staged_counts[kStagedExperts];
-  __shared__ int rep_of_edge[kWave];
+  constexpr int WE = GM * DM < WL ? (GM * DM < 8 ? 8 : GM * DM) : WL;  // ... an edge
+  constexpr int KG = ROWS == 1 ? 4 : 16;   // normalised counts a lane prefetches for the output (and loop unrolling)
+  constexpr int kStaged = ROWS * WAVES <= 4 ? 2048 : 768;   // counts one LP keeps in LDS for its gathers
+  __shared__ float staged_all[ROWS * WAVES][kStaged];
+  __shared__ int rep_of_edge_all[kWave * WAVES];
+  int *rep_of_edge = rep_of_edge_all + threadIdx.x / kWave * kWave;
 
-  const int lane = threadIdx.x;
+  // `lane` is the position inside this LP's lanes, `lane0` the wave lane where they start.
+  const int lane = threadIdx.x % WL, lane0 = threadIdx.x % kWave - lane;
   const int G = EXACT ? GM : a.G, D = EXACT ? DM : a.D;
   const int C = a.C, n = G * D, n_fixed = a.n_fixed;
   const int L = D * C + n_fixed, P = L + D * C;
-  const int grp = blockIdx.x % a.n_group, inst = blockIdx.x / a.n_group;
+  // A wave whose last rows have no LP left repeats the last one and discards the result.
+  const int n_units = a.n_units;
+  const int unit_raw = blockIdx.x * (ROWS * WAVES) + threadIdx.x / WL;
+  const bool unit_on = unit_raw < n_units;
+  const int unit = unit_on ? unit_raw : n_units - 1;
+  const int grp = unit % a.n_group, inst = unit / a.n_group;
+  float *staged_counts = staged_all[threadIdx.x / WL];
+  auto gather = [&](auto v, int src) { return bpermute(v, lane0 + src); };
   const int32_t *__restrict__ wl = a.workload + (int64_t)inst * a.n_experts;
   const int32_t *__restrict__ p2l = a.phy2log + (int64_t)grp * G * P;
   const bool is_edge = lane < n, is_rank = lane < G;
   const int ek = is_edge ? lane / D : 0;   // original rank of my edge
   const int ed = is_edge ? lane % D : 0;   // its replica slot
-  // Up to kStagedExperts counts are staged in LDS as floats, so that the gathers
+  // Up to kStaged counts are staged in LDS as floats, so that the gathers
   // through phy2log do not need a second round trip to global memory.
-  const bool staged = a.n_experts <= kStagedExperts;
+  const bool staged = a.n_experts <= kStaged;
   auto count_of = [&](int e) -> float {
     if (e < 0 || e >= a.n_experts)
       return 0.0f;
@@ -132,8 +206,8 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   // ---- all global reads up front, as independent loads ----
   // (a) the maximum over all experts of all groups, minilp.cu:181-189
   float wmax = 0.0f;
-#pragma unroll 4
-  for (int i = lane; i < a.n_experts; i += kWave) {
+#pragma unroll KG
+  for (int i = lane; i < a.n_experts; i += WL) {
     const float cnt = (float)wl[i];
     wmax = fmaxf(wmax, cnt);
     if (staged)
@@ -160,7 +234,7 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   int out_cnt[KG];
 #pragma unroll
   for (int u = 0; u < KG; ++u) {
-    const int i = lane + u * kWave;
+    const int i = lane + u * WL;
     out_cnt[u] = (a.gw_out && i < G * L) ? wl[grp * G * L + i] : 0;
   }
   __builtin_amdgcn_wave_barrier();   // staged counts are visible to the whole wave
@@ -169,7 +243,7 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
 #pragma unroll
   for (int u = 0; u < KB; ++u)
     fixed_cnt[u] = count_of(fixed_e[u]);
-  wmax = reduce_max<kWave>(wmax);
+  wmax = lp_max<ROWS, WL>(wmax);
 
   LPLB_STAMP(1);
   // ---- per-edge constants (lane j < n): w_j, minilp.cu:203-221 ----
@@ -178,14 +252,14 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     for (int c = 1; c < C; ++c)
       w += count_of(p2l[ek * P + c * D + ed]) / wmax;
   // rank that holds the copy of each edge: invert r2o through LDS
-  rep_of_edge[lane] = ek;
+  rep_of_edge[lane0 + lane] = ek;
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int d = 0; d < DM; ++d)
     if (is_rank && d < D)
-      rep_of_edge[r2o_row[d] * D + d] = lane;
+      rep_of_edge[lane0 + r2o_row[d] * D + d] = lane;
   __builtin_amdgcn_wave_barrier();
-  const int erep = rep_of_edge[lane];
+  const int erep = rep_of_edge[lane0 + lane];
 
   LPLB_STAMP(2);
   // ---- per-rank constants (lane i < G) ----
@@ -202,8 +276,8 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     src[d] = on ? lane * D + d : 0;
     src[DM + d] = on ? r2o_row[d] * D + d : 0;
     // cross-lane reads stay outside lane-dependent conditions
-    const int other = bpermute(erep, src[d]);
-    const float w_own = bpermute(w, src[d]), w_copy = bpermute(w, src[DM + d]);
+    const int other = gather(erep, src[d]);
+    const float w_own = gather(w, src[d]), w_copy = gather(w, src[DM + d]);
     oth[d] = on ? other : lane;
     oth[DM + d] = on ? r2o_row[d] : lane;
     w_e[d] = on ? w_own : 0.0f;
@@ -232,7 +306,7 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   if (T >= 2) part += dpp<kQuadSwap1>(part);
   if (T >= 4) part += dpp<kQuadSwap2>(part);
   if (T >= 8) part += dpp<kHalfMirror>(part);
-  const float part_of_rank = bpermute(part, (lane * T) & (kWave - 1));
+  const float part_of_rank = gather(part, (lane * T) & (WL - 1));
   const float b = is_rank ? -part_of_rank : 0.0f;
   // Big-M column, minilp.cu:275-281: b_i minus the other entries of row i.
   float m = b;
@@ -260,14 +334,14 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     const float wu = w * u;
     const float ao = wu * so, ar = wu * sr;
     const float lam = w * ao * sr;             // w^2 so sr / (so + sr)
-    const float sigma = reduce_sum<WE>(u);
+    const float sigma = lp_sum<ROWS, WE>(u);
     const float kappa = sM * __builtin_amdgcn_rcpf(1.0f + sM * sigma);
 
     float q = 0.0f, lam_e[NE], lam_sum = ss;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float q_own = bpermute(ao, src[d]), q_copy = bpermute(ar, src[DM + d]);
-      const float l_own = bpermute(lam, src[d]), l_copy = bpermute(lam, src[DM + d]);
+      const float q_own = gather(ao, src[d]), q_copy = gather(ar, src[DM + d]);
+      const float l_own = gather(lam, src[d]), l_copy = gather(lam, src[DM + d]);
       // an inactive slot or a self-loop (oth == lane) contributes nothing to S;
       // an inactive slot contributes nothing to q either
       q += slot_on[d] ? q_own + q_copy : 0.0f;
@@ -282,15 +356,15 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     double S[GM];
     const double dst = (double)st, dkv = (double)kappa * (double)v;
     const float st_col = is_rank ? st : 0.0f;
-#pragma unroll
-    for (int c = 0; c < GM; ++c) {
+    static_for<GM>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
       float t = diag_mask[c] * lam_sum;
 #pragma unroll
       for (int e = 0; e < NE; ++e)
         t = __builtin_fmaf(mask[e][c], lam_e[e], t);
-      const double base = EXACT ? dst : (double)readlane(st_col, c) * row_on;
-      S[c] = __builtin_fma(dkv, (double)readlane(v, c), base) + (double)t;
-    }
+      const double base = EXACT ? dst : (double)lp_bcast<ROWS, c>(st_col) * row_on;
+      S[c] = __builtin_fma(dkv, (double)lp_bcast<ROWS, c>(v), base) + (double)t;
+    });
     double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
 
     if (step == 0) LPLB_STAMP(6);
@@ -300,28 +374,28 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     // c before they are scaled, so those broadcasts do not wait for the pivot's
     // reciprocal.  S is symmetric positive definite: no pivoting.
     double my_pivot = 1.0;
-#pragma unroll
-    for (int c = 0; c < GM; ++c) {
-      const double pivot = readlane(S[c], c);
+    static_for<GM>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      const double pivot = lp_bcast<ROWS, c>(S[c]);
       const double rinv = rcp_f64(pivot);
       my_pivot = (lane == c) ? pivot : my_pivot;
       const double f = (lane != c) ? S[c] * rinv : 0.0;   // multiple of row c to subtract from my row
-      rhs = __builtin_fma(-f, readlane(rhs, c), rhs);
+      rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
 #pragma unroll
       for (int c2 = c + 1; c2 < GM; ++c2)
-        S[c2] = __builtin_fma(-f, readlane(S[c2], c), S[c2]);
-    }
+        S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+    });
     if (step == 0) LPLB_STAMP(7);
     const float y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
 
     if (step == 0) LPLB_STAMP(8);
     // r = A^T w and the direction d = x (c - r); the edge part of w is
     // z = u (h - kappa u.h + kappa (m.y - 1000)), h = -B^T y.
-    const float yk = bpermute(y, ek), yrep = bpermute(y, erep);
+    const float yk = gather(y, ek), yrep = gather(y, erep);
     const float hp = -w * (so * yk + sr * yrep);
-    const float my = reduce_sum<WR>(m * y);
-    const float sumy = reduce_sum<WR>(y);
-    const float uh = reduce_sum<WE>(u * hp);
+    const float my = lp_sum<ROWS, WR>(m * y);
+    const float sumy = lp_sum<ROWS, WR>(y);
+    const float uh = lp_sum<ROWS, WE>(u * hp);
     const float shift = kappa * (my - 1000.0f) - kappa * uh;
     const float z = u * (hp + shift);
     const float sumz = uh + shift * sigma;       // = sum of z over the edges
@@ -338,7 +412,7 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     cand = win_r ? fmaxf(cand, d_r) : cand;
     cand = win_s ? fmaxf(cand, d_s) : cand;
     cand = lane == 0 ? fmaxf(fmaxf(cand, d_t), d_M) : cand;
-    d_max = reduce_max<WE>(cand);
+    d_max = lp_max<ROWS, WE>(cand);
     if (with_zero)
       d_max = fmaxf(d_max, 0.0f);
     const float alpha = (float)(0.999 / (double)d_max);
@@ -357,46 +431,68 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
     float row = xs - xt + m * xM - b;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float a_o = bpermute(xo, src[d]), a_r = bpermute(xr, src[DM + d]);
+      const float a_o = gather(xo, src[d]), a_r = gather(xr, src[DM + d]);
       row += w_e[d] * a_o + w_e[DM + d] * a_r;
     }
     if (is_rank)
       res = fmaxf(res, fabsf(row));
     if (is_edge)
       res = fmaxf(res, fabsf(xo + xr - xM - 1.0f));
-    res = reduce_max<WE>(res);
+    res = lp_max<ROWS, WE>(res);
   }
   const bool ok = (double)d_max < 0.1 && 0.0 <= (double)xM && (double)xM < 1e-4 &&
                   (double)res < 0.05;
-  if (lane == 0 && ok)
-    atomicAdd(a.avail, 1);
-  if (is_edge)
-    a.result[(int64_t)blockIdx.x * n + lane] = ok ? xo : 0.5f;
+  // One atomic per wave: thousands of single increments of one address would
+  // queue up behind each other in L2.
+  const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
+  if (threadIdx.x % kWave == 0 && n_ok > 0)
+    atomicAdd(a.avail, n_ok);
+  if (is_edge && unit_on)
+    a.result[(int64_t)unit * n + lane] = ok ? xo : 0.5f;
   // Normalised counts of this group, for the caller.
-  if (a.gw_out) {
+  if (a.gw_out && unit_on) {
     float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;
 #pragma unroll
     for (int u = 0; u < KG; ++u)
-      if (lane + u * kWave < G * L)
-        gw[lane + u * kWave] = (float)out_cnt[u] / wmax;
-    for (int i = lane + KG * kWave; i < G * L; i += kWave)
+      if (lane + u * WL < G * L)
+        gw[lane + u * WL] = (float)out_cnt[u] / wmax;
+    for (int i = lane + KG * WL; i < G * L; i += WL)
       gw[i] = (float)wl[grp * G * L + i] / wmax;
   }
   LPLB_STAMP(12);
 }
 
-template <int GM, int DM> static void launch_solver(const SolveArgs &a, int n_waves, hipStream_t s) {
-  if (a.G == GM && a.D == DM)
-    launch(solve_groups<GM, DM, true>, dim3(n_waves), dim3(kWave), 0, s, a);
+#ifndef LPLB_PACK_FROM
+#define LPLB_PACK_FROM 256   // pack four LPs into a wave once there are this many
+#endif
+#ifndef LPLB_PACK_WAVES
+#define LPLB_PACK_WAVES 1
+#endif
+
+template <int GM, int DM> static void launch_solver(const SolveArgs &a, hipStream_t s) {
+  const bool exact = a.G == GM && a.D == DM;
+  if constexpr (GM <= kRowLanes && GM * DM <= kRowLanes) {
+    if (a.n_units >= LPLB_PACK_FROM) {
+      constexpr int W = LPLB_PACK_WAVES;
+      const dim3 grid((a.n_units + 4 * W - 1) / (4 * W));
+      if (exact)
+        launch(solve_groups<GM, DM, true, 4, W>, grid, dim3(kWave * W), 0, s, a);
+      else
+        launch(solve_groups<GM, DM, false, 4, W>, grid, dim3(kWave * W), 0, s, a);
+      return;
+    }
+  }
+  if (exact)
+    launch(solve_groups<GM, DM, true, 1, 1>, dim3(a.n_units), dim3(kWave), 0, s, a);
   else
-    launch(solve_groups<GM, DM, false>, dim3(n_waves), dim3(kWave), 0, s, a);
+    launch(solve_groups<GM, DM, false, 1, 1>, dim3(a.n_units), dim3(kWave), 0, s, a);
 }
 
-static int dispatch(const SolveArgs &a, int n_waves, hipStream_t s) {
+static int dispatch(const SolveArgs &a, hipStream_t s) {
   const int G = a.G, D = a.D;
 #define LPLB_CASE(GM, DM)                                                      \
   if (G <= GM && D <= DM) {                                                    \
-    launch_solver<GM, DM>(a, n_waves, s);                                             \
+    launch_solver<GM, DM>(a, s);                                               \
     return LPLB_OK;                                                            \
   }
   LPLB_CASE(8, 1) LPLB_CASE(8, 2) LPLB_CASE(8, 4) LPLB_CASE(8, 8)
@@ -445,7 +541,8 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
 #else
   a.clocks = nullptr;
 #endif
-  int rc = dispatch(a, n_instances * n_group, static_cast<hipStream_t>(stream));
+  a.n_units = n_instances * n_group;
+  int rc = dispatch(a, static_cast<hipStream_t>(stream));
   if (rc != LPLB_OK)
     return rc;
   LPLB_HIP_TRY(hipGetLastError());

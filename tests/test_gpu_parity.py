@@ -210,6 +210,54 @@ def test_solve_batched_matches_single(cuda):
         _compare_solve(shape, inp.phy2log, counts[i], batched[i].cpu().numpy(), gws[i].cpu().numpy(), 1)
 
 
+def _shifted_ring(g, shifts):
+    return np.array([[(i + s) % g for s in shifts] for i in range(g)], np.int32)
+
+
+@pytest.mark.parametrize("name,r2o,ep,n_logical,n_inst", [
+    ("cube8x2", None, 8, 256, 301),                          # exact instantiation, last wave part full
+    ("ring8x1", _shifted_ring(8, [1]), 8, 128, 258),
+    ("ring6x2_padded", _shifted_ring(6, [1, 2]), 6, 60, 257),   # rounded up to the 8 x 2 instantiation
+    ("ring16x1", _shifted_ring(16, [1]), 32, 256, 260),      # two groups per instance
+])
+def test_solve_batched_four_per_wave(cuda, name, r2o, ep, n_logical, n_inst):
+    """From 256 LPs on, small shapes are solved four to a wave (one per 16-lane row).
+    That kernel must agree with the one-LP-per-wave kernel (batches under 256) and
+    with the oracle, also in a wave that is only partly filled."""
+    from lplb_amd import topology
+    from lplb_amd.mapping import build_redundancy_mapping
+    r2o = topology.CUBE_8P2E if r2o is None else r2o
+    shape = Shape(np.asarray(r2o, np.int32), ep, n_logical, n_logical + np.asarray(r2o).shape[1] * ep)
+    phy2log, _, _ = build_redundancy_mapping(shape.r2o, ep, n_logical, shape.n_physical, None, n_nodes=1)
+    rng = np.random.default_rng(7)
+    skew = rng.uniform(0.05, 0.6, size=(n_inst, 1))
+    counts = (np.clip(rng.standard_normal((n_inst, n_logical)) * skew + 1, 0, None) * 2 ** 12).astype(np.int32)
+    solver = solver_for(shape)
+    d_r2o, d_p2l = dev(shape.r2o, cuda), dev(phy2log, cuda)
+    wl = dev(counts.reshape(n_inst, shape.n_group, shape.G, shape.L), cuda)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    packed, gws = solver.solve_batched(wl, d_r2o, d_p2l, avail, want_global=True)
+    n_ok = int(avail[0])
+    avail.zero_()
+    parts = [solver.solve_batched(wl[i:i + 100], d_r2o, d_p2l, avail) for i in range(0, n_inst, 100)]
+    assert int(avail[0]) == n_ok
+    by_wave = torch.cat(parts)
+    assert packed.shape == by_wave.shape == (n_inst, shape.n_group, shape.G, shape.D)
+    # b_i is summed by a different number of lanes in the two kernels, so the shares differ by
+    # rounding, amplified where the LP is ill-conditioned (a long ring): compare the flows.
+    a, b = packed.cpu().numpy(), by_wave.cpu().numpy()
+    args = (shape.r2o, phy2log, shape.n_group, shape.C)
+    for i in range(n_inst):
+        flow = np.abs(oracle.edge_flows(counts[i], a[i], *args) - oracle.edge_flows(counts[i], b[i], *args)).max()
+        assert flow <= FLOW_TOL * counts[i].sum(), (i, flow)
+    total_ok = 0
+    for i in (0, n_inst // 2, n_inst - 1):
+        o_avail = oracle.solve(counts[i], shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed)[2]
+        _compare_solve(shape, phy2log, counts[i], packed[i].cpu().numpy(), gws[i].cpu().numpy(), o_avail)
+        total_ok += o_avail
+    assert n_ok >= total_ok
+
+
 # ------------------------------------------------------------------ whole plan
 @pytest.mark.parametrize("cfg,mask", [("cpu_ref_ep8", 0.0), ("v3_ep8_cube", 0.05), ("ep16_hypercube", 0.05),
                                       ("ep32_torus", 0.0)])
