@@ -43,6 +43,7 @@ struct SolveArgs {
   int32_t *avail;
   float *result;             // [n_inst][n_group][G][D]
   int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps, n_units;
+  int staged_stride;   // floats of LDS per LP for its counts, 0 = read them from global memory
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
 
@@ -170,9 +171,14 @@ __global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
   constexpr int WR = GM;             // lanes that can hold a rank
   constexpr int WE = GM * DM < WL ? (GM * DM < 8 ? 8 : GM * DM) : WL;  // ... an edge
   constexpr int KG = ROWS == 1 ? 4 : 16;   // normalised counts a lane prefetches for the output (and loop unrolling)
-  constexpr int kStaged = ROWS * WAVES <= 4 ? 2048 : 768;   // counts one LP keeps in LDS for its gathers
-  __shared__ float staged_all[ROWS * WAVES][kStaged];
+  extern __shared__ float staged_all[];   // a.staged_stride floats per LP of this workgroup
   __shared__ int rep_of_edge_all[kWave * WAVES];
+  __shared__ int feasible_in_workgroup;
+  if (WAVES > 1) {
+    if (threadIdx.x == 0)
+      feasible_in_workgroup = 0;
+    __syncthreads();
+  }
   int *rep_of_edge = rep_of_edge_all + threadIdx.x / kWave * kWave;
 
   // `lane` is the position inside this LP's lanes, `lane0` the wave lane where they start.
@@ -186,16 +192,16 @@ __global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
   const bool unit_on = unit_raw < n_units;
   const int unit = unit_on ? unit_raw : n_units - 1;
   const int grp = unit % a.n_group, inst = unit / a.n_group;
-  float *staged_counts = staged_all[threadIdx.x / WL];
+  float *staged_counts = staged_all + threadIdx.x / WL * a.staged_stride;
   auto gather = [&](auto v, int src) { return bpermute(v, lane0 + src); };
   const int32_t *__restrict__ wl = a.workload + (int64_t)inst * a.n_experts;
   const int32_t *__restrict__ p2l = a.phy2log + (int64_t)grp * G * P;
   const bool is_edge = lane < n, is_rank = lane < G;
   const int ek = is_edge ? lane / D : 0;   // original rank of my edge
   const int ed = is_edge ? lane % D : 0;   // its replica slot
-  // Up to kStaged counts are staged in LDS as floats, so that the gathers
+  // When they fit, the counts are staged in LDS as floats, so that the gathers
   // through phy2log do not need a second round trip to global memory.
-  const bool staged = a.n_experts <= kStaged;
+  const bool staged = a.staged_stride > 0;
   auto count_of = [&](int e) -> float {
     if (e < 0 || e >= a.n_experts)
       return 0.0f;
@@ -442,11 +448,19 @@ __global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
   }
   const bool ok = (double)d_max < 0.1 && 0.0 <= (double)xM && (double)xM < 1e-4 &&
                   (double)res < 0.05;
-  // One atomic per wave: thousands of single increments of one address would
-  // queue up behind each other in L2.
+  // Increments of the one counter queue up behind each other in memory (about
+  // 10 ns each), so the waves of a workgroup add up in LDS first.
   const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
-  if (threadIdx.x % kWave == 0 && n_ok > 0)
-    atomicAdd(a.avail, n_ok);
+  if (WAVES == 1) {
+    if (threadIdx.x == 0 && n_ok > 0)
+      atomicAdd(a.avail, n_ok);
+  } else {
+    if (threadIdx.x % kWave == 0 && n_ok > 0)
+      atomicAdd(&feasible_in_workgroup, n_ok);
+    __syncthreads();   // every wave gets here: none leaves early
+    if (threadIdx.x == 0 && feasible_in_workgroup > 0)
+      atomicAdd(a.avail, feasible_in_workgroup);
+  }
   if (is_edge && unit_on)
     a.result[(int64_t)unit * n + lane] = ok ? xo : 0.5f;
   // Normalised counts of this group, for the caller.
@@ -462,30 +476,39 @@ __global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
   LPLB_STAMP(12);
 }
 
-#ifndef LPLB_PACK_FROM
-#define LPLB_PACK_FROM 256   // pack four LPs into a wave once there are this many
-#endif
-#ifndef LPLB_PACK_WAVES
-#define LPLB_PACK_WAVES 1
-#endif
+// How many LPs share a wave and how many waves a workgroup, by batch size:
+//  * up to kLoneWaves LPs: one wave each, alone in its workgroup (lowest latency;
+//    every wave pays its own increment of the feasibility counter);
+//  * more: workgroups of kWaves waves that combine their increments;
+//  * from kPackFrom LPs on, shapes with G <= 16 and G * D <= 16 put four LPs into
+//    each wave, which takes 2 us longer per wave and a quarter of the waves.
+constexpr int kLoneWaves = 64, kWaves = 4, kPackFrom = 1024;
+constexpr int kLdsLimit = 64 * 1024 - 2048;
+
+template <int GM, int DM, bool EXACT, int ROWS, int WAVES>
+static void launch_variant(SolveArgs a, hipStream_t s) {
+  const int per_wg = ROWS * WAVES;
+  const size_t lds = (size_t)per_wg * a.n_experts * sizeof(float);
+  a.staged_stride = lds <= kLdsLimit ? a.n_experts : 0;
+  launch(solve_groups<GM, DM, EXACT, ROWS, WAVES>, dim3((a.n_units + per_wg - 1) / per_wg),
+         dim3(kWave * WAVES), a.staged_stride ? lds : 0, s, a);
+}
+
+template <int GM, int DM, bool EXACT> static void launch_exactness(const SolveArgs &a, hipStream_t s) {
+  if constexpr (GM <= kRowLanes && GM * DM <= kRowLanes) {
+    if (a.n_units >= kPackFrom)
+      return launch_variant<GM, DM, EXACT, 4, kWaves>(a, s);
+  }
+  if (a.n_units > kLoneWaves)
+    return launch_variant<GM, DM, EXACT, 1, kWaves>(a, s);
+  launch_variant<GM, DM, EXACT, 1, 1>(a, s);
+}
 
 template <int GM, int DM> static void launch_solver(const SolveArgs &a, hipStream_t s) {
-  const bool exact = a.G == GM && a.D == DM;
-  if constexpr (GM <= kRowLanes && GM * DM <= kRowLanes) {
-    if (a.n_units >= LPLB_PACK_FROM) {
-      constexpr int W = LPLB_PACK_WAVES;
-      const dim3 grid((a.n_units + 4 * W - 1) / (4 * W));
-      if (exact)
-        launch(solve_groups<GM, DM, true, 4, W>, grid, dim3(kWave * W), 0, s, a);
-      else
-        launch(solve_groups<GM, DM, false, 4, W>, grid, dim3(kWave * W), 0, s, a);
-      return;
-    }
-  }
-  if (exact)
-    launch(solve_groups<GM, DM, true, 1, 1>, dim3(a.n_units), dim3(kWave), 0, s, a);
+  if (a.G == GM && a.D == DM)
+    launch_exactness<GM, DM, true>(a, s);
   else
-    launch(solve_groups<GM, DM, false, 1, 1>, dim3(a.n_units), dim3(kWave), 0, s, a);
+    launch_exactness<GM, DM, false>(a, s);
 }
 
 static int dispatch(const SolveArgs &a, hipStream_t s) {
