@@ -263,6 +263,30 @@ def main() -> None:
         extras["histogram_sweep_us"] = round(float(h_us.mean()), 2)
         extras["histogram_sweep_GBs"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (float(h_us.mean()) * 1e-6) / 1e9, 1)
 
+        # redirect on a batch 16x the sweep (512 MiB in, 512 MiB out): the fixed cost per launch fades
+        big_n, big_slices = 16 * n_idx, 8 * n_sms
+        big_in = [torch.cat([bufs_in[(j + s) % n_buf] for j in range(16)]) for s in (0, 7)]
+        big_out = [torch.empty_like(b) for b in big_in]
+        big_tables = [solver.count_idx(b, big_slices)[1] for b in big_in]
+
+        def redirect_big(i):
+            rc = lib.lplb_map_idx(big_in[i].data_ptr(), o_w.data_ptr(), big_tables[i].data_ptr(), o2r.data_ptr(),
+                                  sweep_p2l.data_ptr(), big_n, 1, G, D, C, P, big_slices, big_out[i].data_ptr(), stream)
+            assert rc == 0
+        for i in (0, 1):
+            redirect_big(i)
+        big_timer = KernelTimer(lib, 12)
+        torch.cuda.synchronize()
+        for r in range(12):
+            big_timer.arm()
+            redirect_big(r % 2)
+        big_us = float(big_timer.times_us(torch).mean())
+        big_timer.close()
+        extras["redirect_16x_sweep_us"] = round(big_us, 2)
+        extras["redirect_16x_sweep_GBs"] = round(big_n * REDIRECT_BYTES_PER_INDEX / (big_us * 1e-6) / 1e9, 1)
+        extras["redirect_16x_sweep_frac_of_peak"] = round(big_n * REDIRECT_BYTES_PER_INDEX / (big_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+        del big_in, big_out, big_tables
+
         # kernels of the plan in isolation, at the plan's own shape
         wl = counts.view(1, G, L)
         gw = torch.empty(1, G, L, dtype=torch.float32, device=dev)

@@ -150,19 +150,28 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
                  lplb_stream_t stream);
 
 /*
- * One batch's whole plan in a single call: lplb_count_idx, lplb_solve and
- * lplb_map_idx chained on `stream`, i.e. what Planner.run does with three
- * extension calls (lplb/planner.py:245-266).
+ * One batch's whole plan in a single call: what Planner.run does with three
+ * extension calls (lplb/planner.py:245-266), with the same results as
+ * lplb_count_idx, lplb_solve and lplb_map_idx chained on `stream`.  Short
+ * batches (up to 131072 indices) of small LP shapes run as ONE kernel launch in
+ * which the workgroups exchange their histogram rows and the LP's result through
+ * memory; everything else runs as the chain of the three entry points' kernels.
  *
  *   global_counts    int32 [n_logical] or NULL.  NULL: the LP is fed this GPU's
  *                    own histogram, as Planner.run does without a process
  *                    group.  Otherwise the counts already summed over all EP
  *                    ranks (what the all-reduce at lplb/planner.py:214-216
  *                    yields).
- *   counts_by_block  int32 [n_blocks, n_logical], out (see lplb_count_idx)
+ *   n_blocks         upper bound on the workgroups used, at least 1
+ *   counts_by_block  int32 [n_blocks, n_logical]: workspace; on return its last
+ *                    row holds this GPU's tokens per expert (the rows above it
+ *                    are unspecified)
  *   global_workload  fp32 [n_logical], out (see lplb_solve)
  *   o_weight         fp32 [n_group, group_size, dup_per_rank], out
  *   out              int64 [n_elements], out (see lplb_map_idx)
+ *
+ * The one-launch form keeps three counters in a per-device array of the library:
+ * plans of one device must be enqueued on one stream (or otherwise not overlap).
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -171,6 +180,23 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
               int n_local_experts, int n_blocks, int32_t *counts_by_block,
               float *global_workload, float *o_weight, int32_t *avail_num,
               int64_t *out, int step_rule, int n_steps, lplb_stream_t stream);
+
+/*
+ * No counterpart in the reference.  enabled = 0 makes lplb_plan always run the
+ * chain of kernels (for callers that overlap plans of one device on several
+ * streams, or that fill the GPU with other resident kernels); 1 (the default)
+ * lets it use the one-launch form where that applies.  Process-wide.
+ */
+int lplb_plan_set_cooperative(int enabled);
+
+/*
+ * No counterpart in the reference.  The workgroups of the one-launch plan wait
+ * for each other with a bounded number of polls; *count receives how many waits
+ * ran out on the current device since the library was loaded (0 in a healthy
+ * run; a plan with a wait that ran out has undefined output).  Synchronous:
+ * copies one int from the device.
+ */
+int lplb_plan_sync_timeouts(int *count);
 
 #ifdef __cplusplus
 }

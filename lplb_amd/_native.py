@@ -38,6 +38,8 @@ _SIGNATURES = {
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "lplb_plan_set_cooperative": (_i, [_i]),
+    "lplb_plan_sync_timeouts": (_i, [_vp]),
     "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
 }
 
@@ -74,6 +76,18 @@ def load() -> ctypes.CDLL:
 
 def exported_symbols() -> list[str]:
     return list(_SIGNATURES)
+
+
+def set_plan_cooperative(enabled: bool) -> None:
+    """Let ``plan`` run short batches as one kernel launch (default) or always as the chain of kernels."""
+    _check(load().lplb_plan_set_cooperative(1 if enabled else 0))
+
+
+def plan_sync_timeouts() -> int:
+    """Waits between workgroups of the one-launch plan that ran out on the current device (0 when healthy)."""
+    count = ctypes.c_int(-1)
+    _check(load().lplb_plan_sync_timeouts(ctypes.byref(count)))
+    return count.value
 
 
 def _check(rc: int) -> None:

@@ -20,7 +20,7 @@
 // Counter rows and running totals are double-buffered by round parity, which
 // leaves one workgroup barrier per round.  Nothing depends on execution order.
 // The modulo of the hash uses a per-expert reciprocal prepared with the tables.
-#include "common.h"
+#include "map_kernel.h"
 
 namespace lplb {
 
@@ -38,34 +38,6 @@ struct MapArgs {
 };
 #define LPLB_MAP_STAMP(k)                                                                      \
   LPLB_STAMP_AT(blockIdx.x == 0 ? a.clocks + 32 : (blockIdx.x == gridDim.x - 1 ? a.clocks + 48 : nullptr), k)
-
-// Per-expert constants of the redirect, one 16-byte LDS read per token.
-struct __attribute__((aligned(16))) ExpertEntry {
-  int32_t total;     // tokens of this expert in the whole index array
-  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1, 0 for total <= 0)
-  int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
-  int32_t original;  // physical slot of the original
-};
-
-// State of one expert inside one wave, one 16-byte LDS read / write per token.
-struct __attribute__((aligned(16))) WaveSlot {
-  int32_t next;             // ordinal of the wave's next token of this expert
-  int32_t unused;
-  unsigned long long bits;  // lanes of the current chunk that hold this expert
-};
-
-// h mod total with C's truncating sign rule; q = mulhi(|h|, magic) is the true
-// quotient or one less.  WRAP: the hash 499 k + 41 may have wrapped to negative.
-template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
-  const uint32_t a = WRAP ? (uint32_t)max(h, -h) : (uint32_t)h;
-  uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
-  r = min(r, r - (uint32_t)x.total);           // one conditional subtract
-  int32_t m = (WRAP && h < 0) ? -(int32_t)r : (int32_t)r;
-  return x.total > 0 ? m : 0;
-}
-
-constexpr int kMaxWaves = 16;
-typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 template <int K, int R, bool WRAP>
 __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
@@ -117,47 +89,27 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   };
   load_pass(begin);
 
-  auto init_entry = [&](int e, int32_t t, int32_t start) {
-    ExpertEntry x;
-    x.total = t;
-    x.magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : (t == 1 ? 0xffffffffu : 0u);
-    x.expected = t;
-    x.original = -1;
-    table[e] = x;
-    replica[e] = -1;
-    carry[e] = start;
-  };
+  const RedirectShape sh{nl, a.n_ranks, a.G, a.D, a.C, a.L, a.P};
   if (e0 < nl)
-    init_entry(e0, t0, s0);
+    init_entry(table, replica, carry, e0, t0, s0);
   for (int e = tid + nt; e < nl; e += nt)
-    init_entry(e, last[e], prev ? prev[e] : 0);
+    init_entry(table, replica, carry, e, last[e], prev ? prev[e] : 0);
   for (int i = tid; i < n_waves * nl; i += nt) {
     slots[i] = WaveSlot{0, 0, 0ull};
     counts[i] = 0;
     counts[n_waves * nl + i] = 0;
   }
   __syncthreads();
-  auto set_original = [&](int e, int le) {
-    if (le >= 0 && le < nl)
-      table[le].original = (e / a.L) * a.P + (e % a.L);
-  };
-  auto set_replica = [&](int ep_rank, int local, int le, float share, int host) {
-    if (le >= 0 && le < nl) {
-      // fp32 product truncated toward zero (saturating, NaN -> 0)
-      table[le].expected = __float2int_rz(share * (float)table[le].total);
-      replica[le] = ((ep_rank / a.G) * a.G + host + 1) * a.P - cd + local;
-    }
-  };
   if (e0 < nl)
-    set_original(e0, le0);
+    set_original(table, sh, e0, le0);
   for (int e = tid + nt; e < nl; e += nt)
-    set_original(e, a.phy2log[(e / a.L) * a.P + (e % a.L)]);
+    set_original(table, sh, e, a.phy2log[(e / a.L) * a.P + (e % a.L)]);
   if (rep0)
-    set_replica(rank0, local0, rle0, share0, host0);
+    set_replica(table, replica, sh, rank0, local0, rle0, share0, host0);
   for (int i = tid + nt; i < a.n_ranks * cd; i += nt) {
     const int ep_rank = i / cd, local = i % cd, d = local % a.D;
-    set_replica(ep_rank, local, a.phy2log[ep_rank * a.P + local], a.o_weight[ep_rank * a.D + d],
-                a.o2r[(ep_rank % a.G) * a.D + d]);
+    set_replica(table, replica, sh, ep_rank, local, a.phy2log[ep_rank * a.P + local],
+                a.o_weight[ep_rank * a.D + d], a.o2r[(ep_rank % a.G) * a.D + d]);
   }
   // (the barrier after the first phase A also publishes the tables)
   LPLB_MAP_STAMP(1);
@@ -206,26 +158,7 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
         // Phase C.
 #pragma unroll
         for (int c = 0; c < K; ++c) {
-          const int e = ev[r][c];
-          const bool valid = e >= 0;
-          if (valid)
-            atomicOr(&mine[e].bits, my_bit);
-          int64_t o = -1;
-          if (valid) {
-            const i32x4 sraw = *reinterpret_cast<const i32x4 *>(&mine[e]);
-            const i32x4 xraw = *reinterpret_cast<const i32x4 *>(&table[e]);
-            const uint32_t peers_lo = (uint32_t)sraw.z, peers_hi = (uint32_t)sraw.w;
-            const int rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
-            const int cnt = __popc(peers_lo) + __popc(peers_hi);
-            const int32_t k = sraw.x + rank;
-            ExpertEntry x;
-            x.total = xraw.x; x.magic = (uint32_t)xraw.y; x.expected = xraw.z; x.original = xraw.w;
-            // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
-            const int32_t h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
-            o = h >= x.expected ? replica[e] : x.original;
-            if (rank == cnt - 1)   // last peer: advance the ordinal, clear the bitmap
-              *reinterpret_cast<i32x4 *>(&mine[e]) = i32x4{k + 1, 0, 0, 0};
-          }
+          const int64_t o = redirect_token<WRAP>(ev[r][c], mine, table, replica, my_bit);
           const int64_t i = round + ((int64_t)wave * K + c) * kWave + lane;
           if (i < end)
             __builtin_nontemporal_store(o, a.out + i);

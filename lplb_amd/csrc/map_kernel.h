@@ -1,0 +1,101 @@
+// Pieces of the logical -> physical redirect shared by the kernels that run it
+// (map.hip: the streaming redirect; plan.hip: the one-launch plan).
+#pragma once
+#include "common.h"
+
+namespace lplb {
+
+// Per-expert constants of the redirect, one 16-byte LDS read per token.
+struct __attribute__((aligned(16))) ExpertEntry {
+  int32_t total;     // tokens of this expert in the whole index array
+  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1, 0 for total <= 0)
+  int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
+  int32_t original;  // physical slot of the original
+};
+
+// State of one expert inside one wave, one 16-byte LDS read / write per token.
+struct __attribute__((aligned(16))) WaveSlot {
+  int32_t next;             // ordinal of the wave's next token of this expert
+  int32_t unused;
+  unsigned long long bits;  // lanes of the current chunk that hold this expert
+};
+
+// h mod total with C's truncating sign rule; q = mulhi(|h|, magic) is the true
+// quotient or one less.  WRAP: the hash 499 k + 41 may have wrapped to negative.
+template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
+  const uint32_t a = WRAP ? (uint32_t)max(h, -h) : (uint32_t)h;
+  uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
+  r = min(r, r - (uint32_t)x.total);           // one conditional subtract
+  int32_t m = (WRAP && h < 0) ? -(int32_t)r : (int32_t)r;
+  return x.total > 0 ? m : 0;
+}
+
+constexpr int kMaxWaves = 16;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+
+// The shapes the table build needs.
+struct RedirectShape {
+  int n_logical, n_ranks, G, D, C, L, P;
+};
+
+// table / replica / first ordinal of expert e: total tokens t, of which `start` lie
+// before this workgroup's slice.  minilp.cu:466-496.
+__device__ inline void init_entry(ExpertEntry *table, int32_t *replica, int32_t *carry, int e, int32_t t,
+                                  int32_t start) {
+  ExpertEntry x;
+  x.total = t;
+  x.magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : (t == 1 ? 0xffffffffu : 0u);
+  x.expected = t;
+  x.original = -1;
+  table[e] = x;
+  replica[e] = -1;
+  carry[e] = start;
+}
+// Physical slot e holds logical expert le as its original.
+__device__ inline void set_original(ExpertEntry *table, const RedirectShape &sh, int e, int le) {
+  if (le >= 0 && le < sh.n_logical)
+    table[le].original = (e / sh.L) * sh.P + (e % sh.L);
+}
+// Replica slot `local` of EP rank ep_rank copies logical expert le, whose original
+// keeps `share` of its tokens; the copy lives on group rank `host`.
+__device__ inline void set_replica(ExpertEntry *table, int32_t *replica, const RedirectShape &sh, int ep_rank,
+                                   int local, int le, float share, int host) {
+  if (le >= 0 && le < sh.n_logical) {
+    // fp32 product truncated toward zero (saturating, NaN -> 0)
+    table[le].expected = __float2int_rz(share * (float)table[le].total);
+    replica[le] = ((ep_rank / sh.G) * sh.G + host + 1) * sh.P - sh.C * sh.D + local;
+  }
+}
+
+// One token of a 64-index chunk: lanes holding the same expert find each other
+// through the wave's 64-bit bitmap for that expert; the rank among those peers is a
+// popcount of lower lanes and the last peer advances the wave's ordinal.  Returns
+// the physical expert (-1 for e < 0).  All lanes of the wave call it together and
+// put a wave barrier between chunks.
+template <bool WRAP>
+__device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntry *table, const int32_t *replica,
+                                         unsigned long long my_bit) {
+  const bool valid = e >= 0;
+  if (valid)
+    atomicOr(&mine[e].bits, my_bit);
+  int64_t o = -1;
+  if (valid) {
+    const i32x4 sraw = *reinterpret_cast<const i32x4 *>(&mine[e]);
+    const i32x4 xraw = *reinterpret_cast<const i32x4 *>(&table[e]);
+    const uint32_t peers_lo = (uint32_t)sraw.z, peers_hi = (uint32_t)sraw.w;
+    const int rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+    const int cnt = __popc(peers_lo) + __popc(peers_hi);
+    const int32_t k = sraw.x + rank;
+    ExpertEntry x;
+    x.total = xraw.x; x.magic = (uint32_t)xraw.y; x.expected = xraw.z; x.original = xraw.w;
+    // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
+    const int32_t h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
+    o = h >= x.expected ? replica[e] : x.original;
+    if (rank == cnt - 1)   // last peer: advance the ordinal, clear the bitmap
+      *reinterpret_cast<i32x4 *>(&mine[e]) = i32x4{k + 1, 0, 0, 0};
+  }
+  return o;
+}
+
+} // namespace lplb

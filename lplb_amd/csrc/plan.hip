@@ -1,11 +1,433 @@
 // Whole plan in one call: histogram -> LP solve -> redirect on one stream.
-// With the global counts supplied the LP does not depend on this GPU's histogram:
-// it is enqueued first and the histogram launch does not wait for it (it still
-// starts after everything the LP launch waited for); prefix and redirect are ordered
-// after both.  Running the LP as a parallel branch of a captured HIP graph (side
-// stream + events) was measured and rejected: 24.6 us per plan against 20.0 us for
-// the plain chain in the graph.
-#include "common.h"
+//
+// Two ways to run it.
+//
+// Chain: the three entry points' kernels one after the other (histogram, scan,
+// LP, redirect).  With the global counts supplied the LP does not depend on this
+// GPU's histogram: it is enqueued first and the histogram launch does not wait for
+// it (it still starts after everything the LP launch waited for).  Running the LP
+// as a parallel branch of a captured HIP graph (side stream + events) was measured
+// and rejected: 24.6 us per plan against 20.0 us for the plain chain in the graph.
+//
+// One launch (plan_in_one_launch): for batches of up to 64 slices of 2048 indices
+// and LP shapes whose registers fit beside a 512- or 1024-thread workgroup.  Every
+// kernel boundary of the chain costs 3-5 us on this GPU although the kernels have
+// 1-3 us of work, and the LP (8 us, one wave) sits on the critical path.  Here one
+// workgroup per slice and one more for the LP run side by side in a single grid:
+//   slice workgroup: load indices -> per-wave LDS histograms -> publish the slice's
+//     histogram row -> wait until all rows are there -> add up the rows (totals and
+//     counts before this slice) -> tables and per-wave starting ordinals -> wait for
+//     the LP's shares -> redirect and store;
+//   LP workgroup: (own-histogram mode: wait for the rows, add them up) -> solve ->
+//     publish the shares.
+// What crosses workgroups (rows, shares, three counters) is written and read with
+// agent-scope atomics, which go through the XCD's L2 to memory; nothing else is
+// shared, so no cache write-back or invalidate is needed.  The grid is far smaller
+// than the GPU (at most 65 workgroups on 256 CUs), so all workgroups are resident
+// and the waits end; each wait is bounded all the same, and a wait that runs out is
+// counted (lplb_plan_sync_timeouts) instead of hanging the GPU.  The counters live
+// in a per-device array of this library; the last workgroup to leave clears them.
+// Launches of this kernel that overlap on one device (different streams) would
+// share them: run plans of one device on one stream, or switch this path off with
+// lplb_plan_set_cooperative(0).
+#include "map_kernel.h"
+#include "solve_kernel.h"
+
+namespace lplb {
+
+constexpr int kSliceIndices = 2048;   // longest slice of the one-launch plan
+constexpr int kMaxSlices = 64;
+constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
+constexpr int kMaxPolls = 1 << 18;    // about 0.3 s of polling before a wait gives up
+
+// [0] slices whose histogram row is published, [1] workgroups that have left,
+// [2] LP shares published, [3] waits that ran out since the library was loaded.
+static __device__ __attribute__((aligned(64))) int g_plan_sync[16];
+static bool g_cooperative = true;
+
+struct PlanArgs {
+  const int64_t *idx;
+  int64_t n, per;
+  int n_slices;
+  const int32_t *o2r, *phy2log;
+  int32_t *rows;     // [n_slices][n_logical] per-slice histograms, exchanged between workgroups
+  int32_t *totals;   // [n_logical] this GPU's tokens per expert, out
+  int64_t *out;
+  RedirectShape sh;
+  SolveArgs solve;   // result = the shares (o_weight); workload is replaced by totals if local_counts
+  int local_counts;
+  int *sync;
+};
+
+__device__ inline int agent_load(const int *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void agent_store(int *p, int v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// One lane polls *word until it reaches `target`; a wait that runs out is counted.
+// Afterwards this CU's L1 and this XCD's L2 drop what they hold of other XCDs'
+// memory, so that the plain (batched) loads that follow the workgroup barrier see
+// what the other workgroups wrote through to memory before they counted up.
+// (Agent-scope atomic loads would see it too, but the compiler issues those one
+// at a time: 16 of them cost 5 us.)
+__device__ inline void wait_for(int *sync, int word, int target) {
+  int polls = 0;
+  while (agent_load(sync + word) < target && ++polls < kMaxPolls)
+    __builtin_amdgcn_s_sleep(2);
+  if (polls >= kMaxPolls)
+    __hip_atomic_fetch_add(sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+// rows[r][e] summed over r = first, first + step, ...: all rows (t) and those before
+// slice `pid` (before).
+__device__ inline void add_up_rows(const int32_t *rows, int n_rows, int nl, int e, int first, int step, int pid,
+                                   int32_t &t, int32_t &before) {
+  t = 0;
+  before = 0;
+  constexpr int kInFlight = 16;   // loads issued before the first is used (clamped addresses, masked values)
+  for (int r0 = first; r0 < n_rows; r0 += kInFlight * step) {
+    int32_t v[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k)
+      v[k] = rows[(int64_t)min(r0 + k * step, n_rows - 1) * nl + e];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      const int r = r0 + k * step;
+      t += r < n_rows ? v[k] : 0;
+      before += r < pid ? v[k] : 0;
+    }
+  }
+}
+
+// The last of the grid's workgroups to leave clears the counters for the next launch.
+__device__ inline void leave(int *sync, int n_workgroups) {
+  const int before = __hip_atomic_fetch_add(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (before == n_workgroups - 1) {
+    agent_store(sync + 0, 0);
+    agent_store(sync + 2, 0);
+    agent_store(sync + 1, 0);
+  }
+}
+
+// LDS of a slice workgroup.
+static size_t plan_lds_bytes(int n_logical, int n_waves) {
+  const size_t groups = (size_t)n_waves * kWave >= (size_t)n_logical ? (size_t)n_waves * kWave / n_logical : 1;
+  return (size_t)n_logical * (sizeof(ExpertEntry) + 4 + 4 + (size_t)n_waves * (sizeof(WaveSlot) + 4) + groups * 8);
+}
+
+// Debug builds: stamps of the first and the last slice workgroup and of the LP's.
+#define LPLB_PLAN_STAMP(k)                                                                     \
+  LPLB_STAMP_AT(a.solve.clocks == nullptr ? nullptr                                            \
+                : blockIdx.x == 0 ? a.solve.clocks + 64                                        \
+                : blockIdx.x == a.n_slices - 1 ? a.solve.clocks + 80                           \
+                : blockIdx.x == a.n_slices ? a.solve.clocks + 96 : nullptr, k)
+
+// K: 64-index chunks per wave.  WAVES: waves per workgroup.
+template <int GM, int DM, bool EXACT, int K, int WAVES>
+__global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  __shared__ int rep_of_edge_all[WAVES * kWave];
+  const int nl = a.sh.n_logical;
+  const int tid = threadIdx.x;
+  constexpr int nt = WAVES * kWave;
+  const int lane = tid % kWave, wave = tid / kWave;
+  const int pid = blockIdx.x;
+  const int n_workgroups = a.n_slices + 1;
+  const int n_groups = nt >= nl ? nt / nl : 1;   // threads per expert when rows are added up
+
+  if (pid == a.n_slices) {
+    // ------------------------------------------------------------ the LP
+    SolveArgs sa = a.solve;
+    LPLB_PLAN_STAMP(0);
+    if (a.local_counts) {
+      if (tid == 0)
+        wait_for(a.sync, 0, a.n_slices);
+      __syncthreads();
+      int32_t *partial = reinterpret_cast<int32_t *>(smem_raw);   // [n_groups][nl], before the LP stages its counts there
+      const int g = nt >= nl ? tid / nl : 0;
+      if (g < n_groups)
+        for (int e = nt >= nl ? tid % nl : tid; e < nl; e += nt >= nl ? nl : nt) {
+          int32_t t, before;
+          add_up_rows(a.rows, a.n_slices, nl, e, g, n_groups, 0, t, before);
+          partial[(size_t)g * nl + e] = t;
+        }
+      __syncthreads();
+      for (int e = tid; e < nl; e += nt) {
+        int32_t t = 0;
+        for (int k = 0; k < n_groups; ++k)
+          t += partial[(size_t)k * nl + e];
+        a.totals[e] = t;
+      }
+      __syncthreads();   // the totals are read back below by other waves of this workgroup
+      sa.workload = a.totals;
+    }
+    LPLB_PLAN_STAMP(1);
+    if (wave < sa.n_units) {
+      float *staged = reinterpret_cast<float *>(smem_raw) + (size_t)wave * sa.staged_stride;
+      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, wave, staged, rep_of_edge_all + wave * kWave);
+      if (lane == 0 && n_ok > 0)
+        atomicAdd(sa.avail, n_ok);
+    }
+    LPLB_PLAN_STAMP(2);
+    __builtin_amdgcn_s_waitcnt(0);   // the shares have left this CU
+    __syncthreads();
+    LPLB_PLAN_STAMP(3);
+    if (tid == 0) {
+      agent_store(a.sync + 2, 1);
+      leave(a.sync, n_workgroups);
+    }
+    return;
+  }
+
+  // --------------------------------------------------------------- a slice
+  ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);              // [nl]
+  WaveSlot *slots = reinterpret_cast<WaveSlot *>(table + nl);                 // [WAVES][nl]
+  int32_t *replica = reinterpret_cast<int32_t *>(slots + (size_t)WAVES * nl); // [nl]
+  int32_t *start = replica + nl;                                              // [nl]
+  int32_t *counts = start + nl;                                               // [WAVES][nl]
+  int32_t *partial = counts + (size_t)WAVES * nl;                             // [2][n_groups][nl]
+  WaveSlot *mine = slots + (size_t)wave * nl;
+  const unsigned long long my_bit = 1ull << lane;
+  const int64_t begin = slice_begin(a.n, a.per, pid);
+  const int64_t end = slice_begin(a.n, a.per, pid + 1);
+
+  LPLB_PLAN_STAMP(0);
+  int32_t ev[K];   // expert ids, -1 for masked / out-of-range / past the end
+#pragma unroll
+  for (int c = 0; c < K; ++c) {
+    const int64_t i = begin + ((int64_t)wave * K + c) * kWave + lane;
+    const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
+    ev[c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
+  }
+  for (int i = tid; i < WAVES * nl; i += nt) {
+    slots[i] = WaveSlot{0, 0, 0ull};
+    counts[i] = 0;
+  }
+  __syncthreads();
+  // tokens per expert in this wave's chunks
+#pragma unroll
+  for (int c = 0; c < K; ++c)
+    if (ev[c] >= 0)
+      atomicAdd(&counts[(size_t)wave * nl + ev[c]], 1);
+  __syncthreads();
+  // this slice's histogram row, for every workgroup to read
+  for (int e = tid; e < nl; e += nt) {
+    int32_t h = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      h += counts[(size_t)w * nl + e];
+    agent_store(a.rows + (int64_t)pid * nl + e, h);
+  }
+  __builtin_amdgcn_s_waitcnt(0);   // the row has left this CU
+  __syncthreads();
+  LPLB_PLAN_STAMP(1);
+  if (tid == 0) {
+    __hip_atomic_fetch_add(a.sync + 0, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    wait_for(a.sync, 0, a.n_slices);
+  }
+  __syncthreads();
+  LPLB_PLAN_STAMP(2);
+  // add up the rows: tokens per expert in the whole batch and before this slice
+  {
+    const int g = nt >= nl ? tid / nl : 0;
+    if (g < n_groups)
+      for (int e = nt >= nl ? tid % nl : tid; e < nl; e += nt >= nl ? nl : nt) {
+        int32_t t, before;
+        add_up_rows(a.rows, a.n_slices, nl, e, g, n_groups, pid, t, before);
+        partial[(size_t)g * nl + e] = t;
+        partial[(size_t)(n_groups + g) * nl + e] = before;
+      }
+  }
+  __syncthreads();
+  LPLB_PLAN_STAMP(6);
+  for (int e = tid; e < nl; e += nt) {
+    int32_t t = 0, before = 0;
+    for (int g = 0; g < n_groups; ++g) {
+      t += partial[(size_t)g * nl + e];
+      before += partial[(size_t)(n_groups + g) * nl + e];
+    }
+    init_entry(table, replica, start, e, t, before);
+    if (pid == 0 && !a.local_counts)
+      a.totals[e] = t;
+  }
+  __syncthreads();
+  for (int e = tid; e < nl; e += nt)
+    set_original(table, a.sh, e, a.phy2log[(e / a.sh.L) * a.sh.P + (e % a.sh.L)]);
+  LPLB_PLAN_STAMP(7);
+  // each wave's starting ordinals: tokens before this slice + those of the waves before it
+  for (int e = lane; e < nl; e += kWave) {
+    int32_t run = start[e];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      run += w < wave ? counts[(size_t)w * nl + e] : 0;
+    mine[e].next = run;
+  }
+  // the LP's shares decide how many tokens stay on the original
+  LPLB_PLAN_STAMP(3);
+  if (tid == 0)
+    wait_for(a.sync, 2, 1);
+  __syncthreads();
+  LPLB_PLAN_STAMP(4);
+  const int cd = a.sh.C * a.sh.D;
+  for (int i = tid; i < a.sh.n_ranks * cd; i += nt) {
+    const int ep_rank = i / cd, local = i % cd, d = local % a.sh.D;
+    const float share = __hip_atomic_load(a.solve.result + ep_rank * a.sh.D + d, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    set_replica(table, replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local], share,
+                a.o2r[(ep_rank % a.sh.G) * a.sh.D + d]);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < K; ++c) {
+    const int64_t o = redirect_token<false>(ev[c], mine, table, replica, my_bit);
+    const int64_t i = begin + ((int64_t)wave * K + c) * kWave + lane;
+    if (i < end)
+      __builtin_nontemporal_store(o, a.out + i);
+    __builtin_amdgcn_wave_barrier();
+  }
+  LPLB_PLAN_STAMP(5);
+  if (tid == 0)
+    leave(a.sync, n_workgroups);
+}
+
+template <int GM, int DM, bool EXACT, int K, int WAVES>
+static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t s) {
+  if (lds > 64 * 1024) {
+    static hipError_t raised =
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&plan_in_one_launch<GM, DM, EXACT, K, WAVES>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kPlanLdsLimit);
+    if (raised != hipSuccess)
+      return raised;
+  }
+  launch(plan_in_one_launch<GM, DM, EXACT, K, WAVES>, dim3(a.n_slices + 1), dim3(WAVES * kWave), lds, s, a);
+  return hipGetLastError();
+}
+
+// LP shapes the one-launch plan is built for, in the order they are tried, and the
+// workgroup size that leaves the LP its registers: 128 VGPRs per lane at 16 waves,
+// 256 at 8.
+constexpr int kPlanShapes[][2] = {{8, 1}, {8, 2}, {8, 4}, {16, 1}, {16, 2}};
+constexpr int plan_waves(int gm, int dm) { return (gm * dm <= 16 && gm <= 16) ? 16 : 8; }
+static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
+  for (const auto &shape : kPlanShapes)
+    if (G <= shape[0] && D <= shape[1]) {
+      *gm = shape[0];
+      *dm = shape[1];
+      return true;
+    }
+  return false;
+}
+
+template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanArgs &a, hipStream_t s) {
+  constexpr int W = plan_waves(GM, DM);
+  const int64_t chunks = (a.per + kWave - 1) / kWave;
+  const int k = (int)((chunks + W - 1) / W);
+  const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, W);
+  const size_t lds_lp = (size_t)a.solve.n_units * a.solve.n_experts * sizeof(float);
+  a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
+  if (k <= 1)
+    return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s);
+  if (k <= 2)
+    return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds_slices, s);
+  return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s);
+}
+
+// Per-device address of the counters and CU count, looked up once.
+static int plan_device_state(int **sync, int *n_cus) {
+  static int *sync_of[64];
+  static int cus_of[64];
+  int dev = -1;
+  LPLB_HIP_TRY(hipGetDevice(&dev));
+  LPLB_REQUIRE(dev >= 0 && dev < 64, LPLB_EUNSUPPORTED, "plan: device ordinal %d", dev);
+  if (!sync_of[dev]) {
+    int *p = nullptr;
+    LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_plan_sync)));
+    LPLB_HIP_TRY(hipDeviceGetAttribute(&cus_of[dev], hipDeviceAttributeMultiprocessorCount, dev));
+    sync_of[dev] = p;
+  }
+  *sync = sync_of[dev];
+  *n_cus = cus_of[dev];
+  return LPLB_OK;
+}
+
+// Tries the one-launch plan.  *done = false: shape or size outside what it covers.
+static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t *counts, const int32_t *r2o,
+                          const int32_t *o2r, const int32_t *phy2log, int n_group, int G, int D, int C, int P,
+                          int n_blocks, int32_t *counts_by_block, float *global_workload, float *o_weight,
+                          int32_t *avail_num, int64_t *out, int step_rule, int n_steps, hipStream_t s,
+                          bool *done) {
+  *done = false;
+  const int L = P - D * C, n_fixed = L - D * C;
+  const int n_logical = n_group * G * L;
+  if (!g_cooperative || n_elements <= 0 || n_elements > (int64_t)kMaxSlices * kSliceIndices || n_blocks < 2)
+    return LPLB_OK;
+  int gm = 0, dm = 0;
+  if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || global_workload == nullptr)
+    return LPLB_OK;
+  const int waves = plan_waves(gm, dm);
+  // slices of 1024 indices while 64 of them cover the batch, at most n_blocks - 1
+  // (the caller's bound on parallelism; the last row of its table takes the totals)
+#ifndef LPLB_PLAN_FIRST_SLICE
+#define LPLB_PLAN_FIRST_SLICE 1024
+#endif
+  int64_t slices = (n_elements + LPLB_PLAN_FIRST_SLICE - 1) / LPLB_PLAN_FIRST_SLICE;
+  if (slices > kMaxSlices)
+    slices = (n_elements + kSliceIndices - 1) / kSliceIndices;
+  if (slices > n_blocks - 1)
+    slices = n_blocks - 1;
+  const int64_t per = slice_len(n_elements, (int)slices);
+  if (per > (int64_t)waves * 4 * kWave || plan_lds_bytes(n_logical, waves) > (size_t)kPlanLdsLimit)
+    return LPLB_OK;
+  int *sync = nullptr, n_cus = 0;
+  int rc = plan_device_state(&sync, &n_cus);
+  if (rc != LPLB_OK)
+    return rc;
+  if (slices + 1 > n_cus / 2)
+    return LPLB_OK;
+
+  PlanArgs a;
+  a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices;
+  a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block;
+  a.totals = counts_by_block + (int64_t)(n_blocks - 1) * n_logical; a.out = out;
+  a.sh = RedirectShape{n_logical, n_group * G, G, D, C, L, P};
+  a.local_counts = counts == nullptr; a.sync = sync;
+  SolveArgs &sa = a.solve;
+  sa.workload = counts; sa.gw_out = global_workload; sa.r2o = r2o; sa.phy2log = phy2log;
+  sa.avail = avail_num; sa.result = o_weight; sa.n_group = n_group; sa.G = G; sa.D = D; sa.C = C;
+  sa.n_fixed = n_fixed; sa.n_experts = n_logical; sa.step_rule = step_rule; sa.n_steps = n_steps;
+  sa.n_units = n_group; sa.staged_stride = 0; sa.publish_result = 1;
+  sa.clocks = debug_clocks();
+
+  hipError_t err = hipErrorInvalidValue;
+#define LPLB_PLAN_CASE(GM, DM)                                                                 \
+  if (gm == GM && dm == DM)                                                                    \
+    err = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true>(a, s)                        \
+                               : launch_plan_shape<GM, DM, false>(a, s);
+  LPLB_PLAN_CASE(8, 1) LPLB_PLAN_CASE(8, 2) LPLB_PLAN_CASE(8, 4) LPLB_PLAN_CASE(16, 1) LPLB_PLAN_CASE(16, 2)
+#undef LPLB_PLAN_CASE
+  LPLB_HIP_TRY(err);
+  *done = true;
+  return LPLB_OK;
+}
+
+} // namespace lplb
+
+extern "C" int lplb_plan_set_cooperative(int enabled) {
+  lplb::g_cooperative = enabled != 0;
+  return LPLB_OK;
+}
+
+extern "C" int lplb_plan_sync_timeouts(int *count) {
+  using namespace lplb;
+  LPLB_REQUIRE(count != nullptr, LPLB_EINVAL, "plan_sync_timeouts: null pointer");
+  int *sync = nullptr, n_cus = 0;
+  int rc = plan_device_state(&sync, &n_cus);
+  if (rc != LPLB_OK)
+    return rc;
+  LPLB_HIP_TRY(hipMemcpy(count, sync + 3, sizeof(int), hipMemcpyDeviceToHost));
+  return LPLB_OK;
+}
 
 extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
                          const int32_t *global_counts, const int32_t *r2o,
@@ -25,13 +447,23 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
                "plan: n_local_experts=%d does not fit %d x %d replicas", n_local_experts,
                dup_per_rank, n_combined_experts);
   LPLB_REQUIRE(counts_by_block != nullptr, LPLB_EINVAL, "plan: null counts_by_block");
+  LPLB_REQUIRE(n_elements >= 0 && n_elements <= INT32_MAX && (idx || n_elements == 0), LPLB_EINVAL,
+               "plan: bad idx / n_elements=%lld", (long long)n_elements);
+  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL, "plan: idx must be 16-byte aligned");
+  LPLB_REQUIRE(r2o && o2r && phy2log && o_weight && avail_num && (out || n_elements == 0), LPLB_EINVAL,
+               "plan: null pointer");
+  LPLB_REQUIRE(step_rule == LPLB_STEP_REFERENCE_WINDOW || step_rule == LPLB_STEP_FULL_MAX, LPLB_EINVAL,
+               "plan: unknown step_rule %d", step_rule);
+  LPLB_REQUIRE(n_steps >= 0, LPLB_EINVAL, "plan: n_steps=%d", n_steps);
   const int n_logical = n_group * group_size * L;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int rc;
+  bool done = false;
+  int rc = try_one_launch(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
+                          n_combined_experts, n_local_experts, n_blocks, counts_by_block, global_workload,
+                          o_weight, avail_num, out, step_rule, n_steps, s, &done);
+  if (rc != LPLB_OK || done)
+    return rc;
   if (global_counts) {
-    LPLB_REQUIRE(n_elements >= 0 && n_elements <= INT32_MAX && (idx || n_elements == 0), LPLB_EINVAL,
-                 "plan: bad idx / n_elements=%lld", (long long)n_elements);
-    LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL, "plan: idx must be 16-byte aligned");
     rc = lplb_solve(global_counts, global_workload, r2o, phy2log, n_group, group_size, dup_per_rank,
                     n_combined_experts, n_fixed, avail_num, o_weight, step_rule, n_steps, stream);
     if (rc != LPLB_OK)

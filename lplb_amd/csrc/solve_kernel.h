@@ -1,0 +1,479 @@
+// LP solver, device side: one wave64 per EP group (or four small LPs per wave), no
+// workgroup barriers.  Included by the kernels that run it (solve.hip, plan.hip).
+//
+// Problem (reference: minilp.cu:199-293).  For a group of G ranks with D replica
+// slots each, n = G*D replica edges.  Edge j = (k, d) carries the normalised
+// token count w_j of rank k's d-th replicated expert set; a copy lives on the
+// rank i with r2o[i][d] == k.  Variables: x_o[j] (share kept on k), x_r[j] (share
+// sent to the copy), slack s_i per rank, the maximum load t and a Big-M
+// artificial x_M.  Constraints: per rank i,
+//     sum_{j on i} w_j x_o[j] + sum_{j copied to i} w_j x_r[j] + s_i - t + m_i x_M = b_i,
+// per edge x_o[j] + x_r[j] - x_M = 1; minimise t + 1000 x_M.  m makes x = 1 feasible.
+//
+// Method (reference: minilp.cu:331-400): a fixed number of primal affine-scaling
+// steps x <- x (1 - alpha d), d = x (c - A^T w), (A X^2 A^T) w = A X^2 c,
+// alpha = 0.999 / d_max, then a feasibility test; same iteration count, step
+// rule, thresholds and fallback as the reference.
+//
+// What is different is how (A X^2 A^T) w = A X^2 c is solved.  The reference
+// forms the dense (G+n) x (G+n) matrix and calls a block Cholesky.  A has two
+// structural non-zeros per edge column, so eliminating the n edge rows by hand
+// (they are diagonal plus a rank-one term) leaves a G x G system
+//     S = sum_j lambda_j (e_k - e_i)(e_k - e_i)^T + diag(s^2) + t^2 11^T + kappa v v^T
+// -- a weighted graph Laplacian of the replica topology plus a diagonal and two
+// rank-one terms -- with right-hand side -t^2 1 + 1000 kappa v, where
+//     E_j = x_o^2 + x_r^2, u_j = 1/E_j, lambda_j = w_j^2 x_o^2 x_r^2 u_j,
+//     kappa = x_M^2 / (1 + x_M^2 sum u), q = B u, v = m + q.
+// Lane i of the wave owns rank i and row i of S, lane j owns edge j.  S is
+// assembled and [S | rhs] reduced by Gauss-Jordan elimination (pivots and pivot-row
+// entries broadcast with v_readlane, every lane updating its own row) in fp64: the
+// system is tiny, and fp64 here removes the 1e-4..1e-3 rounding scatter a 32-bit
+// factorisation shows on nearly balanced loads.  Everything else is fp32.
+#pragma once
+#include "common.h"
+#include <type_traits>
+#include <utility>
+
+namespace lplb {
+
+
+struct SolveArgs {
+  const int32_t *workload;   // [n_inst][n_experts]
+  float *gw_out;             // [n_inst][n_experts] or null
+  const int32_t *r2o;        // [G][D]
+  const int32_t *phy2log;    // [n_group][G][P]
+  int32_t *avail;
+  float *result;             // [n_inst][n_group][G][D]
+  int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps, n_units;
+  int staged_stride;   // floats of LDS per LP for its counts, 0 = read them from global memory
+  int publish_result;  // 1: a.result is read by other workgroups of the same launch (write-through stores)
+  long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
+};
+
+// Stamps of the first wave (debug builds only).
+#define LPLB_STAMP(k) LPLB_STAMP_AT(blockIdx.x == 0 ? a.clocks : nullptr, k)
+
+template <int CTRL> __device__ inline float dpp(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+constexpr int kQuadSwap1 = 0xB1;    // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;    // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141;  // reverse within 8 lanes
+constexpr int kRowMirror = 0x140;   // reverse within 16 lanes
+
+// Sum of lanes [0, W) (W = 8, 16, 32 or 64; lanes beyond W may hold anything for
+// W < 64 as long as whole 16-lane rows are either inside or outside).  The result
+// is wave-uniform.
+template <int W> __device__ inline float reduce_sum(float v) {
+  v += dpp<kQuadSwap1>(v);
+  v += dpp<kQuadSwap2>(v);
+  v += dpp<kHalfMirror>(v);
+  if (W <= 8)
+    return readlane(v, 0);
+  v += dpp<kRowMirror>(v);
+  if (W <= 16)
+    return readlane(v, 0);
+  if (W <= 32)
+    return readlane(v, 0) + readlane(v, 16);
+  return (readlane(v, 0) + readlane(v, 16)) + (readlane(v, 32) + readlane(v, 48));
+}
+// Max with fmaxf semantics (NaN ignored unless everything is NaN).
+template <int W> __device__ inline float reduce_max(float v) {
+  v = fmaxf(v, dpp<kQuadSwap1>(v));
+  v = fmaxf(v, dpp<kQuadSwap2>(v));
+  v = fmaxf(v, dpp<kHalfMirror>(v));
+  if (W <= 8)
+    return readlane(v, 0);
+  v = fmaxf(v, dpp<kRowMirror>(v));
+  if (W <= 16)
+    return readlane(v, 0);
+  if (W <= 32)
+    return fmaxf(readlane(v, 0), readlane(v, 16));
+  return fmaxf(fmaxf(readlane(v, 0), readlane(v, 16)), fmaxf(readlane(v, 32), readlane(v, 48)));
+}
+
+// 1/a in fp64: hardware estimate (about 2^-23) + one Newton step.
+__device__ inline double rcp_f64(double a) {
+  double r = __builtin_amdgcn_rcp(a);
+  return __builtin_fma(__builtin_fma(-a, r, 1.0), r, r);
+}
+
+// Calls f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>):
+// a loop whose index is a constant expression, as the DPP controls need.
+template <typename F, int... I> __device__ inline void static_for_impl(F &f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ inline void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// ---- one LP per wave (ROWS == 1) or one LP per 16-lane DPP row (ROWS == 4) ----
+// With ROWS == 4 a lane's position inside its row plays the part of the lane id,
+// broadcasts are row-local DPP moves (row_newbcast) and reductions stop at the
+// row, so four independent LPs share the wave's instruction stream.
+constexpr int kRowLanes = 16;
+template <int ROWS> struct Layout {
+  static constexpr int kWidth = ROWS == 1 ? kWave : kRowLanes;   // lanes that serve one LP
+};
+
+template <int LANE> __device__ inline float row_bcast(float v) { return dpp<0x150 + LANE>(v); }
+template <int LANE> __device__ inline double row_bcast(double v) {
+  int2 p = __builtin_bit_cast(int2, v);
+  p.x = __builtin_amdgcn_update_dpp(0, p.x, 0x150 + LANE, 0xF, 0xF, false);
+  p.y = __builtin_amdgcn_update_dpp(0, p.y, 0x150 + LANE, 0xF, 0xF, false);
+  return __builtin_bit_cast(double, p);
+}
+// Value of `v` in lane LANE of this LP's lanes.
+template <int ROWS, int LANE, typename T> __device__ inline T lp_bcast(T v) {
+  if constexpr (ROWS == 1)
+    return readlane(v, LANE);
+  else
+    return row_bcast<LANE>(v);
+}
+// Reductions over the first W lanes of this LP (W <= 16 when ROWS == 4).
+template <int ROWS, int W> __device__ inline float lp_sum(float v) {
+  if constexpr (ROWS == 1) {
+    return reduce_sum<W>(v);
+  } else {
+    v += dpp<kQuadSwap1>(v);
+    v += dpp<kQuadSwap2>(v);
+    v += dpp<kHalfMirror>(v);
+    if (W > 8)
+      v += dpp<kRowMirror>(v);
+    return row_bcast<0>(v);
+  }
+}
+template <int ROWS, int W> __device__ inline float lp_max(float v) {
+  if constexpr (ROWS == 1) {
+    return reduce_max<W>(v);
+  } else {
+    v = fmaxf(v, dpp<kQuadSwap1>(v));
+    v = fmaxf(v, dpp<kQuadSwap2>(v));
+    v = fmaxf(v, dpp<kHalfMirror>(v));
+    if (W > 8)
+      v = fmaxf(v, dpp<kRowMirror>(v));
+    return row_bcast<0>(v);
+  }
+}
+
+
+// A plain store, or one that other workgroups of the running kernel can read back
+// with an agent-scope load (it is written through this XCD's L2).
+__device__ inline void publish(float *p, float v, int through) {
+  if (through)
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else
+    *p = v;
+}
+
+// GM, DM: register-array sizes (group size and replica slots rounded up).
+// EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
+// constant; otherwise rows and columns G..GM-1 of the normal-equation system are
+// padded with the identity, which keeps the factorisation free of branches.
+// ROWS: LPs per wave (1, or 4 when GM <= 16 and GM * DM <= 16).
+//
+// Called by all 64 lanes of a wave; waves share nothing and never synchronise.
+//   first_unit     LP (instance * n_group + group) of the wave's first row
+//   staged_counts  LDS, ROWS * a.staged_stride floats (unused if the stride is 0)
+//   rep_of_edge    LDS, kWave ints
+// Returns how many of the wave's LPs passed the feasibility test (same value in
+// every lane); the caller adds it to a.avail.
+template <int GM, int DM, bool EXACT, int ROWS>
+__device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged_counts_of_wave,
+                               int *rep_of_edge) {
+  constexpr int WL = Layout<ROWS>::kWidth;   // lanes of one LP
+  static_assert(ROWS == 1 || (ROWS == 4 && GM <= kRowLanes && GM * DM <= kRowLanes), "an LP must fit its lanes");
+  constexpr int T = WL / GM;         // lanes that share the work of one rank's b_i
+  constexpr int NE = 2 * DM;         // replica edges that touch one rank
+  constexpr int KB = ROWS == 1 ? 4 : 16;   // fixed-expert counts a lane prefetches for b_i
+  constexpr int WR = GM;             // lanes that can hold a rank
+  constexpr int WE = GM * DM < WL ? (GM * DM < 8 ? 8 : GM * DM) : WL;  // ... an edge
+  constexpr int KG = ROWS == 1 ? 4 : 16;   // normalised counts a lane prefetches for the output (and loop unrolling)
+  const int wave_lane = threadIdx.x % kWave;
+
+  // `lane` is the position inside this LP's lanes, `lane0` the wave lane where they start.
+  const int lane = wave_lane % WL, lane0 = wave_lane - lane;
+  const int G = EXACT ? GM : a.G, D = EXACT ? DM : a.D;
+  const int C = a.C, n = G * D, n_fixed = a.n_fixed;
+  const int L = D * C + n_fixed, P = L + D * C;
+  // A wave whose last rows have no LP left repeats the last one and discards the result.
+  const int n_units = a.n_units;
+  const int unit_raw = first_unit + wave_lane / WL;
+  const bool unit_on = unit_raw < n_units;
+  const int unit = unit_on ? unit_raw : n_units - 1;
+  const int grp = unit % a.n_group, inst = unit / a.n_group;
+  float *staged_counts = staged_counts_of_wave + wave_lane / WL * a.staged_stride;
+  auto gather = [&](auto v, int src) { return bpermute(v, lane0 + src); };
+  const int32_t *__restrict__ wl = a.workload + (int64_t)inst * a.n_experts;
+  const int32_t *__restrict__ p2l = a.phy2log + (int64_t)grp * G * P;
+  const bool is_edge = lane < n, is_rank = lane < G;
+  const int ek = is_edge ? lane / D : 0;   // original rank of my edge
+  const int ed = is_edge ? lane % D : 0;   // its replica slot
+  // When they fit, the counts are staged in LDS as floats, so that the gathers
+  // through phy2log do not need a second round trip to global memory.
+  const bool staged = a.staged_stride > 0;
+  auto count_of = [&](int e) -> float {
+    if (e < 0 || e >= a.n_experts)
+      return 0.0f;
+    return staged ? staged_counts[e] : (float)wl[e];
+  };
+
+  LPLB_STAMP(0);
+  // ---- all global reads up front, as independent loads ----
+  // (a) the maximum over all experts of all groups, minilp.cu:181-189
+  float wmax = 0.0f;
+#pragma unroll KG
+  for (int i = lane; i < a.n_experts; i += WL) {
+    const float cnt = (float)wl[i];
+    wmax = fmaxf(wmax, cnt);
+    if (staged)
+      staged_counts[i] = cnt;
+  }
+  // (b) my edge's experts: raw count of the first, the rest in the loop below
+  const int e_first = (is_edge && C > 0) ? p2l[ek * P + ed] : -1;
+  // (c) the experts of "my" rank that cannot move (T lanes share a rank)
+  const int br = lane / T, bsub = lane % T;
+  int fixed_e[KB];
+#pragma unroll
+  for (int u = 0; u < KB; ++u) {
+    const int j = bsub + u * T;
+    fixed_e[u] = (br < G && j < n_fixed) ? p2l[br * P + D * C + j] : -1;
+  }
+  // (d) topology row of my rank
+  int r2o_row[DM];
+#pragma unroll
+  for (int d = 0; d < DM; ++d) {
+    int k = (is_rank && d < D) ? a.r2o[lane * D + d] : 0;
+    r2o_row[d] = k < 0 ? 0 : (k >= G ? G - 1 : k);
+  }
+  // (e) this group's counts, for the normalised-count output at the end
+  int out_cnt[KG];
+#pragma unroll
+  for (int u = 0; u < KG; ++u) {
+    const int i = lane + u * WL;
+    out_cnt[u] = (a.gw_out && i < G * L) ? wl[grp * G * L + i] : 0;
+  }
+  __builtin_amdgcn_wave_barrier();   // staged counts are visible to the whole wave
+  const float w_first = count_of(e_first);
+  float fixed_cnt[KB];
+#pragma unroll
+  for (int u = 0; u < KB; ++u)
+    fixed_cnt[u] = count_of(fixed_e[u]);
+  wmax = lp_max<ROWS, WL>(wmax);
+
+  LPLB_STAMP(1);
+  // ---- per-edge constants (lane j < n): w_j, minilp.cu:203-221 ----
+  float w = is_edge && C > 0 ? w_first / wmax : 0.0f;
+  if (is_edge)
+    for (int c = 1; c < C; ++c)
+      w += count_of(p2l[ek * P + c * D + ed]) / wmax;
+  // rank that holds the copy of each edge: invert r2o through LDS
+  rep_of_edge[lane0 + lane] = ek;
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int d = 0; d < DM; ++d)
+    if (is_rank && d < D)
+      rep_of_edge[lane0 + r2o_row[d] * D + d] = lane;
+  __builtin_amdgcn_wave_barrier();
+  const int erep = rep_of_edge[lane0 + lane];
+
+  LPLB_STAMP(2);
+  // ---- per-rank constants (lane i < G) ----
+  // Edge e < DM: my own edge (i, e), other end = where its copy lives.
+  // Edge DM + d: the edge copied into my slot d, other end = its original rank.
+  // An inactive edge points at myself, which makes all its terms vanish.
+  int src[NE], oth[NE];
+  float w_e[NE];
+  bool slot_on[DM];
+#pragma unroll
+  for (int d = 0; d < DM; ++d) {
+    const bool on = is_rank && d < D;
+    slot_on[d] = on;
+    src[d] = on ? lane * D + d : 0;
+    src[DM + d] = on ? r2o_row[d] * D + d : 0;
+    // cross-lane reads stay outside lane-dependent conditions
+    const int other = gather(erep, src[d]);
+    const float w_own = gather(w, src[d]), w_copy = gather(w, src[DM + d]);
+    oth[d] = on ? other : lane;
+    oth[DM + d] = on ? r2o_row[d] : lane;
+    w_e[d] = on ? w_own : 0.0f;
+    w_e[DM + d] = on ? w_copy : 0.0f;
+  }
+  // Selectors for assembling my row of S: 1 on my own column, -1 on the column
+  // of each edge's other end.
+  float mask[NE][GM], diag_mask[GM];
+#pragma unroll
+  for (int c = 0; c < GM; ++c) {
+    diag_mask[c] = (lane == c) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int e = 0; e < NE; ++e)
+      mask[e][c] = (oth[e] == c) ? -1.0f : 0.0f;
+  }
+
+  LPLB_STAMP(3);
+  // b_i = -(load of the experts that cannot move), minilp.cu:223-234
+  float part = 0.0f;
+#pragma unroll
+  for (int u = 0; u < KB; ++u)
+    part += fixed_cnt[u] / wmax;
+  if (br < G)
+    for (int j = bsub + KB * T; j < n_fixed; j += T)
+      part += count_of(p2l[br * P + D * C + j]) / wmax;
+  if (T >= 2) part += dpp<kQuadSwap1>(part);
+  if (T >= 4) part += dpp<kQuadSwap2>(part);
+  if (T >= 8) part += dpp<kHalfMirror>(part);
+  const float part_of_rank = gather(part, (lane * T) & (WL - 1));
+  const float b = is_rank ? -part_of_rank : 0.0f;
+  // Big-M column, minilp.cu:275-281: b_i minus the other entries of row i.
+  float m = b;
+#pragma unroll
+  for (int e = 0; e < NE; ++e)
+    m -= w_e[e];
+  m = (m - 1.0f) + 1.0f;
+  if (!is_rank)
+    m = 0.0f;
+
+  LPLB_STAMP(4);
+  // ---- affine scaling ----
+  float xo = 1.0f, xr = 1.0f, xs = 1.0f, xt = 1.0f, xM = 1.0f;
+  float d_max = 0.0f;
+  const int NV = 2 * n + G + 2;
+  const int win_lo = a.step_rule == LPLB_STEP_REFERENCE_WINDOW ? (NV > 32 ? NV - 32 : 0) : 0;
+  const bool with_zero = a.step_rule != LPLB_STEP_REFERENCE_WINDOW || NV < 32;
+  const bool win_o = is_edge && lane >= win_lo, win_r = is_edge && n + lane >= win_lo;
+  const bool win_s = is_rank && 2 * n + lane >= win_lo;
+  const double row_on = is_rank ? 1.0 : 0.0;
+
+  for (int step = 0; step < a.n_steps; ++step) {
+    const float so = xo * xo, sr = xr * xr, ss = xs * xs, st = xt * xt, sM = xM * xM;
+    const float u = is_edge ? __builtin_amdgcn_rcpf(so + sr) : 0.0f;
+    const float wu = w * u;
+    const float ao = wu * so, ar = wu * sr;
+    const float lam = w * ao * sr;             // w^2 so sr / (so + sr)
+    const float sigma = lp_sum<ROWS, WE>(u);
+    const float kappa = sM * __builtin_amdgcn_rcpf(1.0f + sM * sigma);
+
+    float q = 0.0f, lam_e[NE], lam_sum = ss;
+#pragma unroll
+    for (int d = 0; d < DM; ++d) {
+      const float q_own = gather(ao, src[d]), q_copy = gather(ar, src[DM + d]);
+      const float l_own = gather(lam, src[d]), l_copy = gather(lam, src[DM + d]);
+      // an inactive slot or a self-loop (oth == lane) contributes nothing to S;
+      // an inactive slot contributes nothing to q either
+      q += slot_on[d] ? q_own + q_copy : 0.0f;
+      lam_e[d] = (oth[d] == lane) ? 0.0f : l_own;
+      lam_e[DM + d] = (oth[DM + d] == lane) ? 0.0f : l_copy;
+      lam_sum += lam_e[d] + lam_e[DM + d];
+    }
+    const float v = is_rank ? m + q : 0.0f;
+
+    if (step == 0) LPLB_STAMP(5);
+    // Row `lane` of S and its right-hand side, fp64.
+    double S[GM];
+    const double dst = (double)st, dkv = (double)kappa * (double)v;
+    const float st_col = is_rank ? st : 0.0f;
+    static_for<GM>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      float t = diag_mask[c] * lam_sum;
+#pragma unroll
+      for (int e = 0; e < NE; ++e)
+        t = __builtin_fmaf(mask[e][c], lam_e[e], t);
+      const double base = EXACT ? dst : (double)lp_bcast<ROWS, c>(st_col) * row_on;
+      S[c] = __builtin_fma(dkv, (double)lp_bcast<ROWS, c>(v), base) + (double)t;
+    });
+    double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
+
+    if (step == 0) LPLB_STAMP(6);
+    // Gauss-Jordan elimination of [S | rhs] by columns: lane i owns row i, column c
+    // is cleared in every other row at once, so no triangular solves (and no
+    // transposed factor) are needed afterwards.  Row c's entries are read from lane
+    // c before they are scaled, so those broadcasts do not wait for the pivot's
+    // reciprocal.  S is symmetric positive definite: no pivoting.
+    double my_pivot = 1.0;
+    static_for<GM>([&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      const double pivot = lp_bcast<ROWS, c>(S[c]);
+      const double rinv = rcp_f64(pivot);
+      my_pivot = (lane == c) ? pivot : my_pivot;
+      const double f = (lane != c) ? S[c] * rinv : 0.0;   // multiple of row c to subtract from my row
+      rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
+#pragma unroll
+      for (int c2 = c + 1; c2 < GM; ++c2)
+        S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+    });
+    if (step == 0) LPLB_STAMP(7);
+    const float y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
+
+    if (step == 0) LPLB_STAMP(8);
+    // r = A^T w and the direction d = x (c - r); the edge part of w is
+    // z = u (h - kappa u.h + kappa (m.y - 1000)), h = -B^T y.
+    const float yk = gather(y, ek), yrep = gather(y, erep);
+    const float hp = -w * (so * yk + sr * yrep);
+    const float my = lp_sum<ROWS, WR>(m * y);
+    const float sumy = lp_sum<ROWS, WR>(y);
+    const float uh = lp_sum<ROWS, WE>(u * hp);
+    const float shift = kappa * (my - 1000.0f) - kappa * uh;
+    const float z = u * (hp + shift);
+    const float sumz = uh + shift * sigma;       // = sum of z over the edges
+    const float d_o = -xo * (w * yk + z);
+    const float d_r = -xr * (w * yrep + z);
+    const float d_s = -xs * y;
+    const float d_t = xt * (1.0f + sumy);
+    const float d_M = xM * (1000.0f - (my - sumz));
+
+    if (step == 0) LPLB_STAMP(9);
+    // Step length, minilp.cu:354-362.  NaN marks "not in the window".
+    float cand = __builtin_nanf("");
+    cand = win_o ? fmaxf(cand, d_o) : cand;
+    cand = win_r ? fmaxf(cand, d_r) : cand;
+    cand = win_s ? fmaxf(cand, d_s) : cand;
+    cand = lane == 0 ? fmaxf(fmaxf(cand, d_t), d_M) : cand;
+    d_max = lp_max<ROWS, WE>(cand);
+    if (with_zero)
+      d_max = fmaxf(d_max, 0.0f);
+    const float alpha = (float)(0.999 / (double)d_max);
+    xo *= 1.0f - alpha * d_o;
+    xr *= 1.0f - alpha * d_r;
+    xs *= 1.0f - alpha * d_s;
+    xt *= 1.0f - alpha * d_t;
+    xM *= 1.0f - alpha * d_M;
+    if (step == 0) LPLB_STAMP(10);
+  }
+
+  LPLB_STAMP(11);
+  // Feasibility, minilp.cu:369-385.
+  float res = 0.0f;
+  {
+    float row = xs - xt + m * xM - b;
+#pragma unroll
+    for (int d = 0; d < DM; ++d) {
+      const float a_o = gather(xo, src[d]), a_r = gather(xr, src[DM + d]);
+      row += w_e[d] * a_o + w_e[DM + d] * a_r;
+    }
+    if (is_rank)
+      res = fmaxf(res, fabsf(row));
+    if (is_edge)
+      res = fmaxf(res, fabsf(xo + xr - xM - 1.0f));
+    res = lp_max<ROWS, WE>(res);
+  }
+  const bool ok = (double)d_max < 0.1 && 0.0 <= (double)xM && (double)xM < 1e-4 &&
+                  (double)res < 0.05;
+  const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
+  if (is_edge && unit_on)
+    publish(&a.result[(int64_t)unit * n + lane], ok ? xo : 0.5f, a.publish_result);
+  // Normalised counts of this group, for the caller.
+  if (a.gw_out && unit_on) {
+    float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;
+#pragma unroll
+    for (int u = 0; u < KG; ++u)
+      if (lane + u * WL < G * L)
+        gw[lane + u * WL] = (float)out_cnt[u] / wmax;
+    for (int i = lane + KG * WL; i < G * L; i += WL)
+      gw[i] = (float)wl[grp * G * L + i] / wmax;
+  }
+  LPLB_STAMP(12);
+  return n_ok;
+}
+
+} // namespace lplb

@@ -289,6 +289,43 @@ def test_run_matches_oracle_chain(cuda, cfg, mask):
     np.testing.assert_array_equal(out.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("kind", ["empty", "all_masked", "one_token", "odd_length", "one_expert_only"])
+def test_run_edge_inputs(cuda, kind):
+    """Degenerate batches go through the same three kernels (tests/test_idx_processing.py of the
+    reference only draws full random batches; these are the corners it leaves out)."""
+    c = synth.CONFIGS["cpu_ref_ep8"]
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    rng = np.random.default_rng(11)
+    idx = {"empty": np.zeros((0, c.topk), np.int64),
+           "all_masked": np.full((77, c.topk), -1, np.int64),
+           "one_token": rng.integers(0, c.n_logical, size=(1, c.topk), dtype=np.int64),
+           "odd_length": rng.integers(-1, c.n_logical, size=(1237, 1), dtype=np.int64),
+           "one_expert_only": np.full((4096, 1), 5, np.int64)}[kind]
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    phy2log = planner.phy2log.cpu().numpy()
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    n_sms = 16
+    d_idx = dev(idx, cuda)
+    out = planner.run(d_idx, avail, n_sms)
+    torch.cuda.synchronize()
+    assert out.shape == d_idx.shape and out.dtype == torch.int64
+    by_sm = oracle.count_idx(idx.reshape(-1), c.n_logical, n_sms)
+    o_res, _, o_avail = oracle.solve(by_sm[-1], shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed)
+    assert int(avail[0]) == o_avail
+    if kind in ("empty", "all_masked"):
+        assert o_avail == 0 and np.all(o_res == 0.5)      # no tokens: the LP has no scale, fallback shares
+    local, by_sm_gpu = planner.count_workload(d_idx, n_sms)
+    np.testing.assert_array_equal(by_sm_gpu.cpu().numpy(), by_sm)
+    o_weight, _ = planner.solve_probs(local, torch.zeros(1, dtype=torch.int32, device=cuda))
+    want = oracle.map_idx(idx.reshape(-1), o_weight.cpu().numpy(), by_sm, shape.o2r, phy2log, shape.n_group,
+                          shape.C, shape.P).reshape(idx.shape)
+    got = out.cpu().numpy()
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(got == -1, idx == -1)
+    valid = got >= 0
+    np.testing.assert_array_equal(phy2log[got[valid]], idx[valid])   # every token still reaches its expert
+
+
 def test_redirect_full_size_sweep(cuda):
     """[262144 x 8] indices: bit-exact against the oracle, exact split counts, conservation."""
     inp = synth.make_inputs("sweep_redirect")
@@ -343,7 +380,8 @@ def test_plan_entry_point_matches_three_calls(cuda, cfg, use_global):
                                        global_counts=t["counts"] if use_global else None)
     torch.cuda.synchronize()
     want_by_sm = oracle.count_idx(inp.indices, shape.n_logical, n_sms)
-    np.testing.assert_array_equal(by_sm.cpu().numpy(), want_by_sm)
+    # the last row always holds this GPU's totals; the rows above it are the library's workspace
+    np.testing.assert_array_equal(by_sm[-1].cpu().numpy(), want_by_sm[-1])
     workload = inp.global_counts if use_global else want_by_sm[-1]
     avail2 = torch.zeros(1, dtype=torch.int32, device=cuda)
     ref_w, _ = solver.solve(dev(workload.reshape(shape.n_group, shape.G, shape.L), cuda), t["r2o"], t["phy2log"], avail2)
@@ -351,6 +389,40 @@ def test_plan_entry_point_matches_three_calls(cuda, cfg, use_global):
     want = oracle.map_idx(inp.indices, o_weight.cpu().numpy(), want_by_sm, shape.o2r, inp.phy2log, shape.n_group,
                           shape.C, shape.P)
     np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("cfg", ["cpu_ref_ep8", "v3_ep8_cube", "ep16_hypercube", "ep32_torus"])
+@pytest.mark.parametrize("use_global", [True, False])
+@pytest.mark.parametrize("tokens,n_sms", [(None, 256), (37, 256), (4100, 9), (16384, 40), (20000, 256)])
+def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
+    """Short batches run as one kernel launch whose workgroups exchange histogram rows and the
+    LP's shares through memory; the result must be the chain's, bit for bit, call after call."""
+    from lplb_amd import _native
+    inp = synth.make_inputs(cfg, tokens=tokens, mask_fraction=0.05) if tokens else synth.make_inputs(cfg, mask_fraction=0.05)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    solver = solver_for(shape)
+    t = dict(idx=dev(inp.indices, cuda), r2o=dev(shape.r2o, cuda), o2r=dev(shape.o2r, cuda),
+             phy2log=dev(inp.phy2log, cuda), counts=dev(inp.global_counts, cuda))
+    counts = t["counts"] if use_global else None
+    runs = {}
+    try:
+        for mode in (False, True, True):
+            _native.set_plan_cooperative(mode)
+            avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+            out, o_weight, by_sm = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, n_sms,
+                                               global_counts=counts)
+            torch.cuda.synchronize()
+            got = (out.cpu().numpy(), o_weight.cpu().numpy(), by_sm[-1].cpu().numpy(), int(avail[0]))
+            if mode not in runs:
+                runs[mode] = got
+            for a, b in zip(got, runs[False]):
+                np.testing.assert_array_equal(a, b)
+    finally:
+        _native.set_plan_cooperative(True)
+    assert _native.plan_sync_timeouts() == 0
+    np.testing.assert_array_equal(runs[True][2], np.bincount(inp.indices[inp.indices >= 0].ravel(),
+                                                             minlength=c.n_logical))
 
 
 def test_planner_run_equals_plan_with_local_counts(cuda):
