@@ -41,8 +41,10 @@ constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kerne
 constexpr int kMaxPolls = 1 << 18;    // about 0.3 s of polling before a wait gives up
 
 // [0] slices whose histogram row is published, [1] workgroups that have left,
-// [2] LP shares published, [3] waits that ran out since the library was loaded.
-static __device__ __attribute__((aligned(64))) int g_plan_sync[16];
+// [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
+// shares as 8-byte words (1 << 32) | float bits, 0 = not there yet.
+constexpr int kSharesAt = 16, kMaxShares = 256;
+static __device__ __attribute__((aligned(64))) int g_plan_sync[kSharesAt + 2 * kMaxShares];
 static bool g_cooperative = true;
 
 struct PlanArgs {
@@ -100,12 +102,21 @@ __device__ inline void add_up_rows(const int32_t *rows, int n_rows, int nl, int 
   }
 }
 
-// The last of the grid's workgroups to leave clears the counters for the next launch.
-__device__ inline void leave(int *sync, int n_workgroups) {
-  const int before = __hip_atomic_fetch_add(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (before == n_workgroups - 1) {
+// Called by a whole workgroup when it is done.  The last of the grid's workgroups
+// to leave clears the counters and the shares for the next launch.
+__device__ inline void leave(int *sync, int n_workgroups, int n_shares) {
+  __shared__ int last_to_leave;
+  if (threadIdx.x == 0)
+    last_to_leave =
+        __hip_atomic_fetch_add(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_workgroups - 1;
+  __syncthreads();
+  if (!last_to_leave)
+    return;
+  unsigned long long *shares = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
+  for (int i = threadIdx.x; i < n_shares; i += blockDim.x)
+    __hip_atomic_store(shares + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) {
     agent_store(sync + 0, 0);
-    agent_store(sync + 2, 0);
     agent_store(sync + 1, 0);
   }
 }
@@ -134,6 +145,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
   const int lane = tid % kWave, wave = tid / kWave;
   const int pid = blockIdx.x;
   const int n_workgroups = a.n_slices + 1;
+  const int n_shares = a.sh.n_ranks * a.sh.D;
   const int n_groups = nt >= nl ? nt / nl : 1;   // threads per expert when rows are added up
 
   if (pid == a.n_slices) {
@@ -170,13 +182,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
         atomicAdd(sa.avail, n_ok);
     }
     LPLB_PLAN_STAMP(2);
-    __builtin_amdgcn_s_waitcnt(0);   // the shares have left this CU
-    __syncthreads();
-    LPLB_PLAN_STAMP(3);
-    if (tid == 0) {
-      agent_store(a.sync + 2, 1);
-      leave(a.sync, n_workgroups);
-    }
+    leave(a.sync, n_workgroups, n_shares);
     return;
   }
 
@@ -263,19 +269,22 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
       run += w < wave ? counts[(size_t)w * nl + e] : 0;
     mine[e].next = run;
   }
-  // the LP's shares decide how many tokens stay on the original
+  // The LP's shares decide how many tokens stay on the original.  Every thread that
+  // needs one polls it itself: value and "valid" arrive in the same 8-byte word.
   LPLB_PLAN_STAMP(3);
-  if (tid == 0)
-    wait_for(a.sync, 2, 1);
-  __syncthreads();
-  LPLB_PLAN_STAMP(4);
   const int cd = a.sh.C * a.sh.D;
+  const unsigned long long *shares = reinterpret_cast<const unsigned long long *>(a.sync + kSharesAt);
   for (int i = tid; i < a.sh.n_ranks * cd; i += nt) {
     const int ep_rank = i / cd, local = i % cd, d = local % a.sh.D;
-    const float share = __hip_atomic_load(a.solve.result + ep_rank * a.sh.D + d, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-    set_replica(table, replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local], share,
-                a.o2r[(ep_rank % a.sh.G) * a.sh.D + d]);
+    unsigned long long word = 0;
+    int polls = 0;
+    while ((word = __hip_atomic_load(shares + ep_rank * a.sh.D + d, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT)) == 0 && ++polls < kMaxPolls)
+      __builtin_amdgcn_s_sleep(2);
+    if (polls >= kMaxPolls)
+      __hip_atomic_fetch_add(a.sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    set_replica(table, replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local],
+                __builtin_bit_cast(float, (uint32_t)word), a.o2r[(ep_rank % a.sh.G) * a.sh.D + d]);
   }
   __syncthreads();
 #pragma unroll
@@ -287,8 +296,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     __builtin_amdgcn_wave_barrier();
   }
   LPLB_PLAN_STAMP(5);
-  if (tid == 0)
-    leave(a.sync, n_workgroups);
+  leave(a.sync, n_workgroups, n_shares);
 }
 
 template <int GM, int DM, bool EXACT, int K, int WAVES>
@@ -363,7 +371,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (!g_cooperative || n_elements <= 0 || n_elements > (int64_t)kMaxSlices * kSliceIndices || n_blocks < 2)
     return LPLB_OK;
   int gm = 0, dm = 0;
-  if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || global_workload == nullptr)
+  if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || n_group * G * D > kMaxShares || global_workload == nullptr)
     return LPLB_OK;
   const int waves = plan_waves(gm, dm);
   // slices of 1024 indices while 64 of them cover the batch, at most n_blocks - 1
@@ -396,7 +404,8 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   sa.workload = counts; sa.gw_out = global_workload; sa.r2o = r2o; sa.phy2log = phy2log;
   sa.avail = avail_num; sa.result = o_weight; sa.n_group = n_group; sa.G = G; sa.D = D; sa.C = C;
   sa.n_fixed = n_fixed; sa.n_experts = n_logical; sa.step_rule = step_rule; sa.n_steps = n_steps;
-  sa.n_units = n_group; sa.staged_stride = 0; sa.publish_result = 1;
+  sa.n_units = n_group; sa.staged_stride = 0;
+  sa.tagged_result = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
   sa.clocks = debug_clocks();
 
   hipError_t err = hipErrorInvalidValue;

@@ -46,7 +46,8 @@ struct SolveArgs {
   float *result;             // [n_inst][n_group][G][D]
   int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps, n_units;
   int staged_stride;   // floats of LDS per LP for its counts, 0 = read them from global memory
-  int publish_result;  // 1: a.result is read by other workgroups of the same launch (write-through stores)
+  unsigned long long *tagged_result;  // or null: a copy of a.result for other workgroups of the same launch,
+                                      // each value written through to memory as (1 << 32) | its bits
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
 
@@ -158,13 +159,13 @@ template <int ROWS, int W> __device__ inline float lp_max(float v) {
 }
 
 
-// A plain store, or one that other workgroups of the running kernel can read back
-// with an agent-scope load (it is written through this XCD's L2).
-__device__ inline void publish(float *p, float v, int through) {
-  if (through)
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  else
-    *p = v;
+// Stores a share, and if asked also the copy other workgroups of the running kernel
+// poll: the high word says "valid", so value and flag arrive in one 8-byte store.
+__device__ inline void store_share(float *p, unsigned long long *tagged, int64_t i, float v) {
+  p[i] = v;
+  if (tagged)
+    __hip_atomic_store(tagged + i, (1ull << 32) | __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // GM, DM: register-array sizes (group size and replica slots rounded up).
@@ -461,7 +462,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
                   (double)res < 0.05;
   const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
   if (is_edge && unit_on)
-    publish(&a.result[(int64_t)unit * n + lane], ok ? xo : 0.5f, a.publish_result);
+    store_share(a.result, a.tagged_result, (int64_t)unit * n + lane, ok ? xo : 0.5f);
   // Normalised counts of this group, for the caller.
   if (a.gw_out && unit_on) {
     float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;
