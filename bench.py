@@ -16,6 +16,7 @@ carries
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -309,6 +310,26 @@ def main() -> None:
                              phy2log.data_ptr(), idx.numel(), 1, G, D, C, P, n_sms, ws["out"].data_ptr(), stream)
         extras["count_p50_us"] = round(pct(event_times_us(count_only, 1000, 100, torch), 50), 2)
         extras["redirect_p50_us"] = round(pct(event_times_us(map_only, 1000, 100, torch), 50), 2)
+
+        # the plan kernel's own duration, the plan fed by this GPU's own histogram (what Planner.run
+        # does without a process group), and the plan as the chain of the three entry points' kernels
+        plan_timer = KernelTimer(lib, 300)
+        for _ in range(300):
+            plan_timer.arm()
+            plan()
+        extras["plan_kernel_us_p50"] = round(pct(plan_timer.times_us(torch), 50), 2)
+        plan_timer.close()
+        local_args = plan_args[:2] + (None,) + plan_args[3:]
+
+        def plan_local():
+            assert lib.lplb_plan(*local_args, stream) == 0
+        extras["plan_local_counts_us_p50"] = round(pct(event_times_us(plan_local, 1000, 100, torch), 50), 2)
+        assert lib.lplb_plan_set_cooperative(0) == 0
+        extras["plan_as_chain_us_p50"] = round(pct(event_times_us(plan, 1000, 100, torch), 50), 2)
+        extras["plan_local_counts_as_chain_us_p50"] = round(pct(event_times_us(plan_local, 1000, 100, torch), 50), 2)
+        assert lib.lplb_plan_set_cooperative(1) == 0
+        timeouts = ctypes.c_int(-1)
+        assert lib.lplb_plan_sync_timeouts(ctypes.byref(timeouts)) == 0 and timeouts.value == 0, timeouts.value
 
         # the same plan replayed from a HIP graph (8 plans per graph): GPU-side cost without launch overhead
         per_graph = 8

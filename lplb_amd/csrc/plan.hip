@@ -38,7 +38,7 @@ namespace lplb {
 constexpr int kSliceIndices = 2048;   // longest slice of the one-launch plan
 constexpr int kMaxSlices = 64;
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
-constexpr int kMaxPolls = 1 << 18;    // about 0.3 s of polling before a wait gives up
+constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait gives up
 
 // [0] slices whose histogram row is published, [1] workgroups that have left,
 // [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
