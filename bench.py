@@ -154,7 +154,7 @@ def main() -> None:
     stream = torch.cuda.current_stream().cuda_stream
     plan_args = (idx.data_ptr(), idx.numel(), counts.data_ptr(), r2o.data_ptr(), o2r.data_ptr(), phy2log.data_ptr(),
                  1, G, D, C, P, n_sms, by0.data_ptr(), ws["global_workload"].data_ptr(), o_w0.data_ptr(),
-                 avail.data_ptr(), out0.data_ptr(), 0, 5)
+                 avail.data_ptr(), out0.data_ptr(), None, 0, 5)
 
     def plan(stream_handle=stream):
         rc = lib.lplb_plan(*plan_args, stream_handle)
@@ -218,7 +218,7 @@ def main() -> None:
     o_w, _ = solver.solve(tables[0][-1].view(1, G, L), r2o, sweep_p2l, avail)
     def redirect(i):
         rc = lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), tables[i].data_ptr(), o2r.data_ptr(),
-                              sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_sms, bufs_out[i].data_ptr(), stream)
+                              sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_sms, bufs_out[i].data_ptr(), None, stream)
         assert rc == 0
 
     reps = args.roofline_reps
@@ -272,7 +272,7 @@ def main() -> None:
 
         def redirect_big(i):
             rc = lib.lplb_map_idx(big_in[i].data_ptr(), o_w.data_ptr(), big_tables[i].data_ptr(), o2r.data_ptr(),
-                                  sweep_p2l.data_ptr(), big_n, 1, G, D, C, P, big_slices, big_out[i].data_ptr(), stream)
+                                  sweep_p2l.data_ptr(), big_n, 1, G, D, C, P, big_slices, big_out[i].data_ptr(), None, stream)
             assert rc == 0
         for i in (0, 1):
             redirect_big(i)
@@ -307,7 +307,7 @@ def main() -> None:
 
         def map_only():
             lib.lplb_map_idx(idx.data_ptr(), ws["o_weight"].data_ptr(), by_plan.data_ptr(), o2r.data_ptr(),
-                             phy2log.data_ptr(), idx.numel(), 1, G, D, C, P, n_sms, ws["out"].data_ptr(), stream)
+                             phy2log.data_ptr(), idx.numel(), 1, G, D, C, P, n_sms, ws["out"].data_ptr(), None, stream)
         extras["count_p50_us"] = round(pct(event_times_us(count_only, 1000, 100, torch), 50), 2)
         extras["redirect_p50_us"] = round(pct(event_times_us(map_only, 1000, 100, torch), 50), 2)
 

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 1
+#define LPLB_ABI_VERSION 2
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -141,13 +141,22 @@ int lplb_solve_batched(const int32_t *workloads, float *global_workloads,
  * token of a block gets which k is unspecified there; here k always follows
  * index order, which makes the output deterministic and independent of
  * n_blocks.  Values outside [-1, n_logical) map to -1.
+ *
+ *   physical_counts  int32 [n_group * group_size * n_local_experts] or NULL, out:
+ *                    tokens per physical expert, i.e. the bincount of `out` that the
+ *                    reference's test computes afterwards
+ *                    (tests/test_idx_processing.py:100-101) and a dispatch needs.
+ *                    It comes from the kernel's tables (the hash is a bijection on
+ *                    [0, total) unless 499 divides total, which has its own closed
+ *                    form), not from another pass over the tokens.  Needs
+ *                    n_elements <= 4303557 (499 k + 41 must not wrap).
  */
 int lplb_map_idx(const int64_t *idx, const float *o_weight,
                  const int32_t *counts_by_block, const int32_t *o2r,
                  const int32_t *phy2log, int64_t n_elements, int n_group,
                  int group_size, int dup_per_rank, int n_combined_experts,
                  int n_local_experts, int n_blocks, int64_t *out,
-                 lplb_stream_t stream);
+                 int32_t *physical_counts, lplb_stream_t stream);
 
 /*
  * One batch's whole plan in a single call: what Planner.run does with three
@@ -169,6 +178,7 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  *   global_workload  fp32 [n_logical], out (see lplb_solve)
  *   o_weight         fp32 [n_group, group_size, dup_per_rank], out
  *   out              int64 [n_elements], out (see lplb_map_idx)
+ *   physical_counts  int32 [n_physical] or NULL, out (see lplb_map_idx)
  *
  * The one-launch form keeps three counters in a per-device array of the library:
  * plans of one device must be enqueued on one stream (or otherwise not overlap).
@@ -179,7 +189,8 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
               int group_size, int dup_per_rank, int n_combined_experts,
               int n_local_experts, int n_blocks, int32_t *counts_by_block,
               float *global_workload, float *o_weight, int32_t *avail_num,
-              int64_t *out, int step_rule, int n_steps, lplb_stream_t stream);
+              int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
+              lplb_stream_t stream);
 
 /*
  * No counterpart in the reference.  enabled = 0 makes lplb_plan always run the

@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1
@@ -37,10 +37,10 @@ _SIGNATURES = {
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
-    "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_plan_set_cooperative": (_i, [_i]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
-    "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
 }
 
 
@@ -193,7 +193,8 @@ class CompiledSolver:
 
     # -- csrc/plugin.cpp:602-660 -------------------------------------------------
     def map_idx(self, mapping_idx: torch.Tensor, o_weight: torch.Tensor, local_workload_split_by_sm: torch.Tensor,
-                o2r: torch.Tensor, phy2log: torch.Tensor, n_sms: int, block_dim: int = 256) -> torch.Tensor:
+                o2r: torch.Tensor, phy2log: torch.Tensor, n_sms: int, block_dim: int = 256,
+                physical_counts: torch.Tensor | None = None) -> torch.Tensor:
         _require(mapping_idx.dtype == torch.int64, "mapping_idx.dtype == int64")
         _require(mapping_idx.is_cuda, "mapping_idx.device().is_cuda()")
         _require(mapping_idx.is_contiguous(), "mapping_idx.is_contiguous()")
@@ -213,19 +214,30 @@ class CompiledSolver:
                  and tuple(by_sm.shape) == (n_sms, self.n_experts),
                  "local_workload_split_by_sm is a contiguous int32 [n_sms, n_experts] GPU tensor")
         _require(block_dim == 256, "slices are aligned to 256 indices")
+        self._check_physical_counts(physical_counts)
         out = torch.empty_like(mapping_idx)
         _check(self.lib.lplb_map_idx(mapping_idx.data_ptr(), o_weight.data_ptr(), by_sm.data_ptr(), o2r.data_ptr(),
                                      phy2log.data_ptr(), mapping_idx.numel(), self.n_group, self.group_size,
                                      self.dup_per_rank, self.n_combined_experts, self.n_local_experts, n_sms,
-                                     out.data_ptr(), _stream(mapping_idx)))
+                                     out.data_ptr(),
+                                     physical_counts.data_ptr() if physical_counts is not None else None,
+                                     _stream(mapping_idx)))
         return out
+
+    def _check_physical_counts(self, t: torch.Tensor | None) -> None:
+        """Optional output of map_idx / plan: tokens per physical expert (the bincount of the result)."""
+        if t is not None:
+            _require(t.dtype == torch.int32 and t.is_cuda and t.is_contiguous()
+                     and t.numel() == self.n_group * self.group_size * self.n_local_experts,
+                     "physical_counts is a contiguous int32 [n_group * group_size * n_local_experts] GPU tensor")
 
     # -- lplb/planner.py:245-266 in one library call -----------------------------
     def plan(self, idx: torch.Tensor, r2o: torch.Tensor, o2r: torch.Tensor, phy2log: torch.Tensor,
              avail_num: torch.Tensor, n_sms: int, global_counts: torch.Tensor | None = None,
-             workspace: dict | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+             workspace: dict | None = None,
+             physical_counts: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         """Histogram, LP solve and redirect of one batch.  Returns (physical indices, o_weight,
-        counts per slice).  ``global_counts`` (int32 [n_logical]) replaces this GPU's own histogram
+        workspace table whose last row holds this GPU's tokens per logical expert).  ``global_counts`` (int32 [n_logical]) replaces this GPU's own histogram
         as the LP's workload.  ``workspace`` may carry preallocated ``out``, ``by_sm``, ``o_weight``
         and ``global_workload`` tensors to reuse."""
         _require(idx.dtype == torch.int64 and idx.is_cuda and idx.is_contiguous(),
@@ -242,6 +254,7 @@ class CompiledSolver:
         if global_counts is not None:
             _require(global_counts.dtype == torch.int32 and global_counts.is_cuda and global_counts.is_contiguous()
                      and global_counts.numel() == self.n_experts, "global_counts is a contiguous int32 [n_experts] GPU tensor")
+        self._check_physical_counts(physical_counts)
         ws = workspace if workspace is not None else {}
         dev = idx.device
         out = ws.get("out")
@@ -262,5 +275,6 @@ class CompiledSolver:
                                   self.group_size, self.dup_per_rank, self.n_combined_experts,
                                   self.n_local_experts, n_sms, by_sm.data_ptr(), gw.data_ptr(),
                                   o_weight.data_ptr(), avail_num.data_ptr(), out.data_ptr(),
+                                  physical_counts.data_ptr() if physical_counts is not None else None,
                                   self.step_rule, self.n_steps, _stream(idx)))
         return out, o_weight, by_sm

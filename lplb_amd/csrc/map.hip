@@ -34,10 +34,17 @@ struct MapArgs {
   int64_t per;
   int n_logical, n_ranks, G, D, C, L, P, n_blocks;
   int64_t *out;
+  int32_t *physical_counts;   // [n_ranks * P] tokens per physical expert, or null
   long long *clocks;   // debug builds: stamps of the first and the last workgroup (else null)
 };
 #define LPLB_MAP_STAMP(k)                                                                      \
   LPLB_STAMP_AT(blockIdx.x == 0 ? a.clocks + 32 : (blockIdx.x == gridDim.x - 1 ? a.clocks + 48 : nullptr), k)
+
+__global__ void zero_ints(int32_t *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    p[i] = 0;
+}
 
 template <int K, int R, bool WRAP>
 __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
@@ -169,6 +176,8 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
       }
     }
   }
+  if (pid == 0 && a.physical_counts)   // the tables are complete since the first barrier
+    emit_physical_counts(table, replica, sh, a.phy2log, a.physical_counts, tid, nt);
   __builtin_amdgcn_s_waitcnt(0);
   LPLB_MAP_STAMP(6);
 }
@@ -198,7 +207,8 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
                             const int32_t *phy2log, int64_t n_elements,
                             int n_group, int group_size, int dup_per_rank,
                             int n_combined_experts, int n_local_experts,
-                            int n_blocks, int64_t *out, lplb_stream_t stream) {
+                            int n_blocks, int64_t *out, int32_t *physical_counts,
+                            lplb_stream_t stream) {
   using namespace lplb;
   LPLB_REQUIRE(n_elements >= 0 && n_elements <= INT32_MAX, LPLB_EINVAL,
                "map_idx: n_elements=%lld out of range", (long long)n_elements);
@@ -212,15 +222,26 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
                n_local_experts, L, dup_per_rank * n_combined_experts);
   LPLB_REQUIRE(o_weight && counts_by_block && o2r && phy2log && (n_elements == 0 || (idx && out)),
                LPLB_EINVAL, "map_idx: null pointer");
-  if (n_elements == 0)
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // 499 k + 41 stays below 2^31 for every ordinal k < n_elements
+  const bool wrap = n_elements > (INT32_MAX - 41) / 499;
+  LPLB_REQUIRE(!(wrap && physical_counts), LPLB_EUNSUPPORTED,
+               "map_idx: physical_counts needs n_elements <= %d", (INT32_MAX - 41) / 499);
+  if (n_elements == 0) {
+    if (physical_counts) {   // a kernel, not a memset: memset nodes misbehave in replayed HIP graphs here
+      const int n_physical = n_group * group_size * n_local_experts;
+      launch(zero_ints, dim3((n_physical + 255) / 256), dim3(256), 0, s, physical_counts, n_physical);
+      LPLB_HIP_TRY(hipGetLastError());
+    }
     return LPLB_OK;
+  }
 
   MapArgs a;
   a.idx = idx; a.o_weight = o_weight; a.by_block = counts_by_block; a.o2r = o2r;
   a.phy2log = phy2log; a.n = n_elements; a.per = slice_len(n_elements, n_blocks);
   a.n_ranks = n_group * group_size; a.n_logical = a.n_ranks * L;
   a.G = group_size; a.D = dup_per_rank; a.C = n_combined_experts; a.L = L;
-  a.P = n_local_experts; a.n_blocks = n_blocks; a.out = out;
+  a.P = n_local_experts; a.n_blocks = n_blocks; a.out = out; a.physical_counts = physical_counts;
 #ifdef LPLB_PHASE_CLOCKS
   a.clocks = g_phase_clocks;
 #else
@@ -239,9 +260,6 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   const int64_t per_wave = (chunks + n_waves - 1) / n_waves;
   const size_t lds = map_lds_bytes(a.n_logical, n_waves);
   const dim3 grid(n_blocks), block(n_waves * kWave);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  // 499 k + 41 stays below 2^31 for every ordinal k < n_elements
-  const bool wrap = n_elements > (INT32_MAX - 41) / 499;
   hipError_t err;
 #define LPLB_MAP_CASE(K, R)                                                                    \
   err = wrap ? launch_redirect<K, R, true>(a, grid, block, lds, s)                             \

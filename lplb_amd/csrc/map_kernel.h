@@ -68,6 +68,41 @@ __device__ inline void set_replica(ExpertEntry *table, int32_t *replica, const R
   }
 }
 
+// How many of an expert's `total` tokens stay on the original:
+// #{k in [0, total) : (499 k + 41) mod total < expected}.  499 is prime, so unless it
+// divides total the hash is a bijection on [0, total) and the answer is expected
+// clamped to [0, total]; if total = 499 m the hash is 499 (k mod m) + 41, each value
+// taken 499 times.  Valid while 499 k + 41 stays below 2^31.
+__device__ inline int32_t kept_on_original(int32_t total, int32_t expected) {
+  if (total <= 0)
+    return 0;
+  const int32_t want = min(max(expected, 0), total);
+  if (total % 499 != 0)
+    return want;
+  const int32_t m = total / 499;
+  return 499 * (want > 41 ? min(m, (want - 41 + 498) / 499) : 0);
+}
+
+// Tokens per physical expert, = bincount of the redirect's output, from the tables
+// of any one workgroup: every slot is the original or the replica of its logical expert.
+__device__ inline void emit_physical_counts(const ExpertEntry *table, const int32_t *replica,
+                                            const RedirectShape &sh, const int32_t *phy2log, int32_t *counts,
+                                            int tid, int nt) {
+  for (int i = tid; i < sh.n_ranks * sh.P; i += nt) {
+    const int le = phy2log[i];
+    int32_t v = 0;
+    if (le >= 0 && le < sh.n_logical) {
+      const ExpertEntry x = table[le];
+      const int32_t kept = kept_on_original(x.total, x.expected);
+      if (x.original == i)
+        v = kept;
+      else if (replica[le] == i)
+        v = x.total - kept;
+    }
+    counts[i] = v;
+  }
+}
+
 // One token of a 64-index chunk: lanes holding the same expert find each other
 // through the wave's 64-bit bitmap for that expert; the rank among those peers is a
 // popcount of lower lanes and the last peer advances the wave's ordinal.  Returns

@@ -55,6 +55,7 @@ struct PlanArgs {
   int32_t *rows;     // [n_slices][n_logical] per-slice histograms, exchanged between workgroups
   int32_t *totals;   // [n_logical] this GPU's tokens per expert, out
   int64_t *out;
+  int32_t *physical_counts;   // [n_ranks * P] tokens per physical expert, or null
   RedirectShape sh;
   SolveArgs solve;   // result = the shares (o_weight); workload is replaced by totals if local_counts
   int local_counts;
@@ -295,6 +296,8 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
       __builtin_nontemporal_store(o, a.out + i);
     __builtin_amdgcn_wave_barrier();
   }
+  if (pid == 0 && a.physical_counts)
+    emit_physical_counts(table, replica, a.sh, a.phy2log, a.physical_counts, tid, nt);
   LPLB_PLAN_STAMP(5);
   leave(a.sync, n_workgroups, n_shares);
 }
@@ -363,8 +366,8 @@ static int plan_device_state(int **sync, int *n_cus) {
 static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t *counts, const int32_t *r2o,
                           const int32_t *o2r, const int32_t *phy2log, int n_group, int G, int D, int C, int P,
                           int n_blocks, int32_t *counts_by_block, float *global_workload, float *o_weight,
-                          int32_t *avail_num, int64_t *out, int step_rule, int n_steps, hipStream_t s,
-                          bool *done) {
+                          int32_t *avail_num, int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
+                          hipStream_t s, bool *done) {
   *done = false;
   const int L = P - D * C, n_fixed = L - D * C;
   const int n_logical = n_group * G * L;
@@ -398,6 +401,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices;
   a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block;
   a.totals = counts_by_block + (int64_t)(n_blocks - 1) * n_logical; a.out = out;
+  a.physical_counts = physical_counts;
   a.sh = RedirectShape{n_logical, n_group * G, G, D, C, L, P};
   a.local_counts = counts == nullptr; a.sync = sync;
   SolveArgs &sa = a.solve;
@@ -444,7 +448,7 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
                          int group_size, int dup_per_rank, int n_combined_experts,
                          int n_local_experts, int n_blocks, int32_t *counts_by_block,
                          float *global_workload, float *o_weight, int32_t *avail_num,
-                         int64_t *out, int step_rule, int n_steps,
+                         int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
                          lplb_stream_t stream) {
   using namespace lplb;
   LPLB_REQUIRE(n_group > 0 && group_size > 0 && dup_per_rank > 0 && n_blocks > 0, LPLB_EINVAL,
@@ -469,7 +473,7 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
   bool done = false;
   int rc = try_one_launch(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
                           n_combined_experts, n_local_experts, n_blocks, counts_by_block, global_workload,
-                          o_weight, avail_num, out, step_rule, n_steps, s, &done);
+                          o_weight, avail_num, out, physical_counts, step_rule, n_steps, s, &done);
   if (rc != LPLB_OK || done)
     return rc;
   if (global_counts) {
@@ -492,5 +496,5 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
   }
   return lplb_map_idx(idx, o_weight, counts_by_block, o2r, phy2log, n_elements, n_group,
                       group_size, dup_per_rank, n_combined_experts, n_local_experts, n_blocks, out,
-                      stream);
+                      physical_counts, stream);
 }

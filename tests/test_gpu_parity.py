@@ -69,11 +69,15 @@ def test_map_idx_matches_oracle(cuda, case, n, n_sms):
     solver = solver_for(shape)
     d_idx = dev(idx, cuda)
     _, by_sm = solver.count_idx(d_idx, n_sms)
-    out = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms)
+    phys = torch.full((shape.n_physical,), -7, dtype=torch.int32, device=cuda)
+    out = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms,
+                         physical_counts=phys)
     torch.cuda.synchronize()
     got = out.cpu().numpy()
     want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
     np.testing.assert_array_equal(got, want)
+    # tokens per physical expert, as the reference's test counts them (tests/test_idx_processing.py:100-101)
+    np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
     # reference test's properties (tests/test_idx_processing.py:88-98)
     assert got.min() >= -1 and got.max() < shape.n_physical
     assert np.array_equal(got == -1, idx == -1)
@@ -108,9 +112,39 @@ def test_map_idx_extreme_weights(cuda):
     solver = solver_for(shape)
     d_idx = dev(idx, cuda)
     _, by_sm = solver.count_idx(d_idx, 64)
-    got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 64).cpu().numpy()
+    phys = torch.empty(shape.n_physical, dtype=torch.int32, device=cuda)
+    got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 64,
+                         physical_counts=phys).cpu().numpy()
     want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
     np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
+
+
+@pytest.mark.parametrize("multiple", [1, 2, 7])
+def test_physical_counts_when_499_divides_a_total(cuda, multiple):
+    """The per-expert hash (499 k + 41) mod total is a bijection unless 499 divides total; then it takes
+    total / 499 values 499 times each and the closed form of the counts changes."""
+    name, r2o, nl, ep, red, reorder, _ = REFERENCE_SOLVE_CASES[0]
+    shape, _, phy2log, _, _ = reference_style_case(r2o, nl, ep, red, True, seed=7)
+    rng = np.random.default_rng(multiple)
+    replicated = [int(phy2log[r * shape.P + s]) for r in range(ep) for s in range(shape.C * shape.D)]
+    counts = rng.integers(1, 300, size=nl)
+    counts[replicated[:6]] = 499 * multiple            # replicated experts with degenerate totals
+    counts[replicated[6]] = 499 * multiple + 1
+    idx = rng.permutation(np.repeat(np.arange(nl, dtype=np.int64), counts))
+    solver = solver_for(shape)
+    d_idx = dev(idx, cuda)
+    _, by_sm = solver.count_idx(d_idx, 32)
+    for trial in range(4):
+        o_weight = rng.uniform(0, 1, size=(shape.n_group, shape.G, shape.D)).astype(np.float32)
+        if trial == 0:
+            o_weight[:] = 41.0 / (499 * multiple)      # expected = 41 (or 40): the first hash value is 41
+        phys = torch.empty(shape.n_physical, dtype=torch.int32, device=cuda)
+        got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 32,
+                             physical_counts=phys).cpu().numpy()
+        want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
 
 
 # -------------------------------------------------------------------- solver
@@ -309,6 +343,12 @@ def test_run_edge_inputs(cuda, kind):
     out = planner.run(d_idx, avail, n_sms)
     torch.cuda.synchronize()
     assert out.shape == d_idx.shape and out.dtype == torch.int64
+    phys = torch.full((c.n_physical,), -7, dtype=torch.int32, device=cuda)
+    out2, _, _ = planner.solver.plan(d_idx, planner.r2o, planner.o2r, planner.phy2log,
+                                     torch.zeros(1, dtype=torch.int32, device=cuda), n_sms, physical_counts=phys)
+    assert torch.equal(out, out2)
+    np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(out.cpu().numpy()[out.cpu().numpy() >= 0].ravel(),
+                                                                  minlength=c.n_physical))
     by_sm = oracle.count_idx(idx.reshape(-1), c.n_logical, n_sms)
     o_res, _, o_avail = oracle.solve(by_sm[-1], shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed)
     assert int(avail[0]) == o_avail
@@ -410,10 +450,12 @@ def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
         for mode in (False, True, True):
             _native.set_plan_cooperative(mode)
             avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+            phys = torch.full((shape.n_physical,), -7, dtype=torch.int32, device=cuda)
             out, o_weight, by_sm = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, n_sms,
-                                               global_counts=counts)
+                                               global_counts=counts, physical_counts=phys)
             torch.cuda.synchronize()
-            got = (out.cpu().numpy(), o_weight.cpu().numpy(), by_sm[-1].cpu().numpy(), int(avail[0]))
+            got = (out.cpu().numpy(), o_weight.cpu().numpy(), by_sm[-1].cpu().numpy(), int(avail[0]),
+                   phys.cpu().numpy())
             if mode not in runs:
                 runs[mode] = got
             for a, b in zip(got, runs[False]):
@@ -423,6 +465,8 @@ def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
     assert _native.plan_sync_timeouts() == 0
     np.testing.assert_array_equal(runs[True][2], np.bincount(inp.indices[inp.indices >= 0].ravel(),
                                                              minlength=c.n_logical))
+    out = runs[True][0]
+    np.testing.assert_array_equal(runs[True][4], np.bincount(out[out >= 0].ravel(), minlength=c.n_physical))
 
 
 def test_planner_run_equals_plan_with_local_counts(cuda):

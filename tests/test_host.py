@@ -190,9 +190,9 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert sorted(_native.exported_symbols()) == declared
-    assert lib.lplb_abi_version() == 1
+    assert lib.lplb_abi_version() == _native.ABI_VERSION == 2
     header = (ROOT / "include" / "lplb_hip.h").read_text()
-    assert "#define LPLB_ABI_VERSION 1" in header
+    assert f"#define LPLB_ABI_VERSION {_native.ABI_VERSION}" in header
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
@@ -209,7 +209,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.lplb_solve(p, p, p, p, 1, 8, 2, 1, 2, p, p, 7, 5, None) == 1    # unknown step rule
     assert lib.lplb_solve(p, None, p, p, 1, 8, 2, 1, 2, p, p, 0, 5, None) == 1
     assert lib.lplb_solve_batched(p, None, p, p, 0, 1, 8, 2, 1, 2, p, p, 0, 5, None) == 1
-    assert lib.lplb_map_idx(p, p, p, p, p, 4, 1, 8, 2, 1, 2, 4, p, None) == 1  # 2 slots per rank cannot hold 2 replicas
-    assert lib.lplb_map_idx(p, p, p, p, None, 4, 1, 8, 2, 1, 34, 4, p, None) == 1
-    assert lib.lplb_plan(p, 4, None, p, p, p, 1, 8, 2, 1, 34, 0, p, p, p, p, p, 0, 5, None) == 1
+    assert lib.lplb_map_idx(p, p, p, p, p, 4, 1, 8, 2, 1, 2, 4, p, None, None) == 1  # 2 slots per rank cannot hold 2 replicas
+    assert lib.lplb_map_idx(p, p, p, p, None, 4, 1, 8, 2, 1, 34, 4, p, None, None) == 1
+    assert lib.lplb_plan(p, 4, None, p, p, p, 1, 8, 2, 1, 34, 0, p, p, p, p, p, None, 0, 5, None) == 1
     assert lib.lplb_copy_calibration(p, p, 3, None) == 1
