@@ -144,19 +144,24 @@ class Planner:
         """
         return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256)
 
-    def run(self, idx: torch.Tensor, avail_counter: torch.Tensor, n_sms: int | None = None) -> torch.Tensor:
+    def run(self, idx: torch.Tensor, avail_counter: torch.Tensor, n_sms: int | None = None, *,
+            physical_counts: torch.Tensor | None = None) -> torch.Tensor:
         """Assign a physical expert to every selected logical expert.
 
         :param idx: int64 logical expert ids, any shape, contiguous, values in [-1, n_logical).
         :param avail_counter: int32 tensor with one element, counts feasible LP solves.
         :param n_sms: number of slices / workgroups; defaults to the GPU's compute-unit count.
+        :param physical_counts: optional int32 [n_routed_experts] output: tokens per physical expert
+            (the bincount of the result, which the reference leaves to the caller).
         """
         if n_sms is None:
             n_sms = torch.cuda.get_device_properties(idx.device).multi_processor_count
         if self.ep_group is None:
             # count_workload -> solve_probs -> weighted_select_target in one library call
-            out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms)
+            out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
+                                                      physical_counts=physical_counts)
             return out
         local_workload, local_workload_by_sm = self.count_workload(idx, n_sms)
         o_weight, _global_workload = self.solve_probs(local_workload, avail_counter)
-        return self.weighted_select_target(idx, o_weight, local_workload_by_sm, n_sms)
+        return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256,
+                                   physical_counts=physical_counts)
