@@ -236,7 +236,7 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
     return LPLB_OK;
   }
 
-  MapArgs a;
+  MapArgs a{};
   a.idx = idx; a.o_weight = o_weight; a.by_block = counts_by_block; a.o2r = o2r;
   a.phy2log = phy2log; a.n = n_elements; a.per = slice_len(n_elements, n_blocks);
   a.n_ranks = n_group * group_size; a.n_logical = a.n_ranks * L;

@@ -43,8 +43,11 @@ constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait 
 // [0] slices whose histogram row is published, [1] workgroups that have left,
 // [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
 // shares as 8-byte words (1 << 32) | float bits, 0 = not there yet.
+// From kTotalsAt on (own-histogram mode), the batch's tokens per logical expert, to
+// which every slice adds its row.
 constexpr int kSharesAt = 16, kMaxShares = 256;
-static __device__ __attribute__((aligned(64))) int g_plan_sync[kSharesAt + 2 * kMaxShares];
+constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
+static __device__ __attribute__((aligned(64))) int g_plan_sync[kTotalsAt + kMaxTotals];
 static bool g_cooperative = true;
 
 struct PlanArgs {
@@ -105,7 +108,7 @@ __device__ inline void add_up_rows(const int32_t *rows, int n_rows, int nl, int 
 
 // Called by a whole workgroup when it is done.  The last of the grid's workgroups
 // to leave clears the counters and the shares for the next launch.
-__device__ inline void leave(int *sync, int n_workgroups, int n_shares) {
+__device__ inline void leave(int *sync, int n_workgroups, int n_shares, int n_totals) {
   __shared__ int last_to_leave;
   if (threadIdx.x == 0)
     last_to_leave =
@@ -116,6 +119,8 @@ __device__ inline void leave(int *sync, int n_workgroups, int n_shares) {
   unsigned long long *shares = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
   for (int i = threadIdx.x; i < n_shares; i += blockDim.x)
     __hip_atomic_store(shares + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int i = threadIdx.x; i < n_totals; i += blockDim.x)
+    agent_store(sync + kTotalsAt + i, 0);
   if (threadIdx.x == 0) {
     agent_store(sync + 0, 0);
     agent_store(sync + 1, 0);
@@ -153,37 +158,48 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     // ------------------------------------------------------------ the LP
     SolveArgs sa = a.solve;
     LPLB_PLAN_STAMP(0);
+    // Own-histogram mode: the LP waves start at once (their table loads do not need
+    // the counts) and pick the counts up from LDS; the wave after them waits for the
+    // slices, fetches the totals the slices have added up in memory and hands them over.
+    __shared__ int counts_ready;
+    float *staged = reinterpret_cast<float *>(smem_raw);
     if (a.local_counts) {
       if (tid == 0)
-        wait_for(a.sync, 0, a.n_slices);
+        counts_ready = 0;
       __syncthreads();
-      int32_t *partial = reinterpret_cast<int32_t *>(smem_raw);   // [n_groups][nl], before the LP stages its counts there
-      const int g = nt >= nl ? tid / nl : 0;
-      if (g < n_groups)
-        for (int e = nt >= nl ? tid % nl : tid; e < nl; e += nt >= nl ? nl : nt) {
-          int32_t t, before;
-          add_up_rows(a.rows, a.n_slices, nl, e, g, n_groups, 0, t, before);
-          partial[(size_t)g * nl + e] = t;
+      sa.counts_ready = &counts_ready;
+      if (wave == sa.n_units) {
+        if (lane == 0)
+          wait_for(a.sync, 0, a.n_slices);
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        for (int e0 = lane; e0 < nl; e0 += 8 * kWave) {
+          int32_t t[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            t[k] = a.sync[kTotalsAt + min(e0 + k * kWave, nl - 1)];
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (e0 + k * kWave < nl) {
+              staged[e0 + k * kWave] = (float)t[k];
+              a.totals[e0 + k * kWave] = t[k];
+            }
         }
-      __syncthreads();
-      for (int e = tid; e < nl; e += nt) {
-        int32_t t = 0;
-        for (int k = 0; k < n_groups; ++k)
-          t += partial[(size_t)k * nl + e];
-        a.totals[e] = t;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0)
+          __hip_atomic_store(&counts_ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
-      __syncthreads();   // the totals are read back below by other waves of this workgroup
-      sa.workload = a.totals;
     }
     LPLB_PLAN_STAMP(1);
     if (wave < sa.n_units) {
-      float *staged = reinterpret_cast<float *>(smem_raw) + (size_t)wave * sa.staged_stride;
-      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, wave, staged, rep_of_edge_all + wave * kWave);
+      // (own-histogram mode: every LP of the batch reads the one staged copy)
+      float *mine = a.local_counts ? staged : staged + (size_t)wave * sa.staged_stride;
+      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, wave, mine, rep_of_edge_all + wave * kWave);
       if (lane == 0 && n_ok > 0)
         atomicAdd(sa.avail, n_ok);
     }
     LPLB_PLAN_STAMP(2);
-    leave(a.sync, n_workgroups, n_shares);
+    leave(a.sync, n_workgroups, n_shares, a.local_counts ? nl : 0);
     return;
   }
 
@@ -225,6 +241,8 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     for (int w = 0; w < WAVES; ++w)
       h += counts[(size_t)w * nl + e];
     agent_store(a.rows + (int64_t)pid * nl + e, h);
+    if (a.local_counts && h != 0)
+      __hip_atomic_fetch_add(a.sync + kTotalsAt + e, h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __builtin_amdgcn_s_waitcnt(0);   // the row has left this CU
   __syncthreads();
@@ -299,7 +317,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
   if (pid == 0 && a.physical_counts)
     emit_physical_counts(table, replica, a.sh, a.phy2log, a.physical_counts, tid, nt);
   LPLB_PLAN_STAMP(5);
-  leave(a.sync, n_workgroups, n_shares);
+  leave(a.sync, n_workgroups, n_shares, a.local_counts ? nl : 0);
 }
 
 template <int GM, int DM, bool EXACT, int K, int WAVES>
@@ -337,6 +355,8 @@ template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanAr
   const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, W);
   const size_t lds_lp = (size_t)a.solve.n_units * a.solve.n_experts * sizeof(float);
   a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
+  if (a.local_counts && a.solve.staged_stride == 0)   // the LP takes its counts from LDS in that mode
+    return hipErrorInvalidValue;
   if (k <= 1)
     return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s);
   if (k <= 2)
@@ -377,6 +397,9 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || n_group * G * D > kMaxShares || global_workload == nullptr)
     return LPLB_OK;
   const int waves = plan_waves(gm, dm);
+  // own-histogram mode: a spare wave beside the LPs, the totals fit the accumulator and the LDS
+  if (counts == nullptr && (n_group >= waves || n_logical > kMaxTotals))
+    return LPLB_OK;
   // slices of 1024 indices while 64 of them cover the batch, at most n_blocks - 1
   // (the caller's bound on parallelism; the last row of its table takes the totals)
 #ifndef LPLB_PLAN_FIRST_SLICE
@@ -397,7 +420,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (slices + 1 > n_cus / 2)
     return LPLB_OK;
 
-  PlanArgs a;
+  PlanArgs a{};   // every field the host does not set below is zero
   a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices;
   a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block;
   a.totals = counts_by_block + (int64_t)(n_blocks - 1) * n_logical; a.out = out;

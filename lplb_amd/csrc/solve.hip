@@ -112,11 +112,11 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
   LPLB_REQUIRE(n_experts > 0 && n_experts <= (1 << 24) && (int64_t)n_instances * n_group <= INT32_MAX,
                LPLB_EINVAL, "solve: %lld experts x %d instances out of range",
                (long long)n_experts, n_instances);
-  SolveArgs a;
+  SolveArgs a{};
   a.workload = workloads; a.gw_out = global_workloads; a.r2o = r2o; a.phy2log = phy2log;
   a.avail = avail_num; a.result = results; a.n_group = n_group; a.G = group_size;
   a.D = dup_per_rank; a.C = n_experts_per_var; a.n_fixed = n_experts_fixed;
-  a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps; a.tagged_result = nullptr;
+  a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps; a.tagged_result = nullptr; a.counts_ready = nullptr;
 #ifdef LPLB_PHASE_CLOCKS
   a.clocks = g_phase_clocks;
 #else

@@ -46,6 +46,8 @@ struct SolveArgs {
   float *result;             // [n_inst][n_group][G][D]
   int n_group, G, D, C, n_fixed, n_experts, step_rule, n_steps, n_units;
   int staged_stride;   // floats of LDS per LP for its counts, 0 = read them from global memory
+  const int *counts_ready;   // or null.  LDS flag: once it is non-zero the caller has put the counts of this
+                             // wave's LP into staged_counts (as floats) and a.workload is not read
   unsigned long long *tagged_result;  // or null: a copy of a.result for other workgroups of the same launch,
                                       // each value written through to memory as (1 << 32) | its bits
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
@@ -222,18 +224,9 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 
   LPLB_STAMP(0);
   // ---- all global reads up front, as independent loads ----
-  // (a) the maximum over all experts of all groups, minilp.cu:181-189
-  float wmax = 0.0f;
-#pragma unroll KG
-  for (int i = lane; i < a.n_experts; i += WL) {
-    const float cnt = (float)wl[i];
-    wmax = fmaxf(wmax, cnt);
-    if (staged)
-      staged_counts[i] = cnt;
-  }
-  // (b) my edge's experts: raw count of the first, the rest in the loop below
+  // (a) my edge's experts: raw count of the first, the rest in the loop below
   const int e_first = (is_edge && C > 0) ? p2l[ek * P + ed] : -1;
-  // (c) the experts of "my" rank that cannot move (T lanes share a rank)
+  // (b) the experts of "my" rank that cannot move (T lanes share a rank)
   const int br = lane / T, bsub = lane % T;
   int fixed_e[KB];
 #pragma unroll
@@ -241,19 +234,44 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     const int j = bsub + u * T;
     fixed_e[u] = (br < G && j < n_fixed) ? p2l[br * P + D * C + j] : -1;
   }
-  // (d) topology row of my rank
+  // (c) topology row of my rank
   int r2o_row[DM];
 #pragma unroll
   for (int d = 0; d < DM; ++d) {
     int k = (is_rank && d < D) ? a.r2o[lane * D + d] : 0;
     r2o_row[d] = k < 0 ? 0 : (k >= G ? G - 1 : k);
   }
-  // (e) this group's counts, for the normalised-count output at the end
-  int out_cnt[KG];
+  // (d) the counts: the maximum over all experts of all groups, minilp.cu:181-189, and
+  // (e) this group's counts, for the normalised-count output at the end.  A caller
+  // that is still producing the counts hands them over in LDS; the table loads
+  // above are on their way meanwhile.
+  const bool prestaged = a.counts_ready != nullptr;
+  float wmax = 0.0f;
+  float out_cnt[KG];
+  if (prestaged) {
+    while (__hip_atomic_load(a.counts_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0)
+      __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    for (int i = lane; i < a.n_experts; i += WL)
+      wmax = fmaxf(wmax, staged_counts[i]);
 #pragma unroll
-  for (int u = 0; u < KG; ++u) {
-    const int i = lane + u * WL;
-    out_cnt[u] = (a.gw_out && i < G * L) ? wl[grp * G * L + i] : 0;
+    for (int u = 0; u < KG; ++u) {
+      const int i = lane + u * WL;
+      out_cnt[u] = (a.gw_out && i < G * L) ? staged_counts[grp * G * L + i] : 0.0f;
+    }
+  } else {
+#pragma unroll KG
+    for (int i = lane; i < a.n_experts; i += WL) {
+      const float cnt = (float)wl[i];
+      wmax = fmaxf(wmax, cnt);
+      if (staged)
+        staged_counts[i] = cnt;
+    }
+#pragma unroll
+    for (int u = 0; u < KG; ++u) {
+      const int i = lane + u * WL;
+      out_cnt[u] = (a.gw_out && i < G * L) ? (float)wl[grp * G * L + i] : 0.0f;
+    }
   }
   __builtin_amdgcn_wave_barrier();   // staged counts are visible to the whole wave
   const float w_first = count_of(e_first);
@@ -469,9 +487,9 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 #pragma unroll
     for (int u = 0; u < KG; ++u)
       if (lane + u * WL < G * L)
-        gw[lane + u * WL] = (float)out_cnt[u] / wmax;
+        gw[lane + u * WL] = out_cnt[u] / wmax;
     for (int i = lane + KG * WL; i < G * L; i += WL)
-      gw[i] = (float)wl[grp * G * L + i] / wmax;
+      gw[i] = count_of(grp * G * L + i) / wmax;
   }
   LPLB_STAMP(12);
   return n_ok;
