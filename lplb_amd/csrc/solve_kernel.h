@@ -407,19 +407,42 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // Gauss-Jordan elimination of [S | rhs] by columns: lane i owns row i, column c
     // is cleared in every other row at once, so no triangular solves (and no
     // transposed factor) are needed afterwards.  Row c's entries are read from lane
-    // c before they are scaled, so those broadcasts do not wait for the pivot's
-    // reciprocal.  S is symmetric positive definite: no pivoting.
+    // c, whose own multiple f is zero.  S is symmetric positive definite: no pivoting.
+    // The only serial chain is pivot -> reciprocal -> f -> entry (c+1, c+1) -> next
+    // pivot; it is written out in that order, with the rest of column step c (which
+    // nothing waits for) placed between the links of the next reciprocal, because
+    // the compiler keeps the order it is given here.
     double my_pivot = 1.0;
+    double pivot = lp_bcast<ROWS, 0>(S[0]);
+    double rinv = rcp_f64(pivot);
     static_for<GM>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
-      const double pivot = lp_bcast<ROWS, c>(S[c]);
-      const double rinv = rcp_f64(pivot);
+      auto clear = [&](auto c2c, double f) {
+        constexpr int c2 = decltype(c2c)::value;
+        if constexpr (c2 < GM)
+          S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+      };
       my_pivot = (lane == c) ? pivot : my_pivot;
       const double f = (lane != c) ? S[c] * rinv : 0.0;   // multiple of row c to subtract from my row
+      double next_pivot = 1.0, estimate = 1.0, error = 0.0;
+      clear(std::integral_constant<int, c + 1>{}, f);
+      if constexpr (c + 1 < GM) {
+        next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
+        estimate = __builtin_amdgcn_rcp(next_pivot);
+      }
       rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
-#pragma unroll
-      for (int c2 = c + 1; c2 < GM; ++c2)
-        S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+      clear(std::integral_constant<int, c + 2>{}, f);
+      if constexpr (c + 1 < GM)
+        error = __builtin_fma(-next_pivot, estimate, 1.0);
+      clear(std::integral_constant<int, c + 3>{}, f);
+      clear(std::integral_constant<int, c + 4>{}, f);
+      if constexpr (c + 1 < GM) {
+        rinv = __builtin_fma(error, estimate, estimate);   // = rcp_f64(next_pivot)
+        pivot = next_pivot;
+      }
+      static_for<(GM > c + 5 ? GM - c - 5 : 0)>([&](auto kk) {
+        clear(std::integral_constant<int, c + 5 + decltype(kk)::value>{}, f);
+      });
     });
     if (step == 0) LPLB_STAMP(7);
     const float y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
