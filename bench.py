@@ -34,7 +34,7 @@ REDIRECT_BYTES_PER_INDEX = 16
 # HBM bytes one redirect launch moves at the sweep shape, from rocprofv3 FETCH_SIZE and WRITE_SIZE (two
 # runs), each scaled by what the same counter reads for the plain copy kernel of known size:
 # 16 797 KiB read + 16 376 KiB written, 1.012 x the algorithmic bytes.
-REDIRECT_TRAFFIC_BYTES_SWEEP = 33_969_000
+REDIRECT_TRAFFIC_BYTES_SWEEP = 34_238_000
 HISTOGRAM_BYTES_PER_INDEX = 8
 
 
@@ -211,14 +211,18 @@ def main() -> None:
     bufs_in = [to_dev(np.roll(flat, int(rng.integers(0, n_idx)))) for _ in range(n_buf)]
     bufs_out = [torch.empty_like(b) for b in bufs_in]
     sweep_p2l = to_dev(sweep.phy2log)
+    # Two slices per CU: at this size two 8-wave workgroups per CU beat one of 16 waves (one's ranking
+    # overlaps the other's loads and stores); the figure with one slice per CU is in the extras.
+    roof_blocks = 2 * n_sms
     tables = []
     for b in bufs_in:
-        total, by = solver.count_idx(b, n_sms)
+        total, by = solver.count_idx(b, roof_blocks)
         tables.append(by)
     o_w, _ = solver.solve(tables[0][-1].view(1, G, L), r2o, sweep_p2l, avail)
-    def redirect(i):
-        rc = lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), tables[i].data_ptr(), o2r.data_ptr(),
-                              sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_sms, bufs_out[i].data_ptr(), None, stream)
+    def redirect(i, n_blocks=roof_blocks, table=None):
+        rc = lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), (table if table is not None else tables[i]).data_ptr(),
+                              o2r.data_ptr(), sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_blocks,
+                              bufs_out[i].data_ptr(), None, stream)
         assert rc == 0
 
     reps = args.roofline_reps
@@ -243,7 +247,8 @@ def main() -> None:
     copy_gbs = alg_bytes / (float(copy_us.mean()) * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": REDIRECT_TRAFFIC_BYTES_SWEEP,
-                "kernel": "redirect_indices", "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64",
+                "kernel": "redirect_indices",
+                "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64, {roof_blocks} slices",
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
                 "p50_launch_us": round(pct(red_us, 50), 2), "distinct_buffer_pairs": n_buf,
                 "copy_kernel_GBs_same_bytes": round(copy_gbs, 1),
@@ -251,9 +256,22 @@ def main() -> None:
     extras["redirect_tokens_per_s"] = round(n_idx / (red_avg * 1e-6), 1)
 
     if not args.skip_extras:
+        # the same redirect with one slice per CU (the reference's default n_sms = SM count)
+        cu_tables = [solver.count_idx(b, n_sms)[1] for b in bufs_in]
+        for i in range(n_buf):
+            redirect(i, n_sms, cu_tables[i])
+        cu_timer = KernelTimer(lib, 4 * n_buf)
+        torch.cuda.synchronize()
+        for _ in range(4):
+            for i in range(n_buf):
+                cu_timer.arm()
+                redirect(i, n_sms, cu_tables[i])
+        extras["redirect_sweep_us_one_slice_per_cu"] = round(float(cu_timer.times_us(torch).mean()), 2)
+        cu_timer.close()
+
         # histogram at the sweep shape (8 B per index)
         def hist(i):
-            rc = lib.lplb_count_idx(bufs_in[i].data_ptr(), n_idx, cfg.n_logical, n_sms, tables[i].data_ptr(), stream)
+            rc = lib.lplb_count_idx(bufs_in[i].data_ptr(), n_idx, cfg.n_logical, n_sms, cu_tables[i].data_ptr(), stream)
             assert rc == 0
         k = [0]
 
@@ -265,7 +283,7 @@ def main() -> None:
         extras["histogram_sweep_GBs"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (float(h_us.mean()) * 1e-6) / 1e9, 1)
 
         # redirect on a batch 16x the sweep (512 MiB in, 512 MiB out): the fixed cost per launch fades
-        big_n, big_slices = 16 * n_idx, 8 * n_sms
+        big_n, big_slices = 16 * n_idx, 4 * n_sms
         big_in = [torch.cat([bufs_in[(j + s) % n_buf] for j in range(16)]) for s in (0, 7)]
         big_out = [torch.empty_like(b) for b in big_in]
         big_tables = [solver.count_idx(b, big_slices)[1] for b in big_in]

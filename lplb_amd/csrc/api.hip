@@ -32,6 +32,20 @@ long long *g_phase_clocks = nullptr;
 
 static thread_local LaunchEvents g_launch_events;
 
+int current_device_cu_count() {
+  static int cus_of[64];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return 0;
+  if (cus_of[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      return 0;
+    cus_of[dev] = n;
+  }
+  return cus_of[dev];
+}
+
 LaunchEvents take_launch_events() {
   const LaunchEvents ev = g_launch_events;
   g_launch_events = LaunchEvents{};

@@ -38,6 +38,9 @@ struct LaunchEvents {
 };
 LaunchEvents take_launch_events();
 
+// Compute units of the current device (looked up once per device); 0 if the query fails.
+int current_device_cu_count();
+
 // Every kernel of the library is launched through here.  If the calling thread
 // armed a pair of events, the launch records the kernel's own begin and end
 // timestamps into them (not the time the launch was enqueued).

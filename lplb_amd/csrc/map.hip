@@ -7,10 +7,10 @@
 // per block but not which token gets which.  Here k is canonical.
 //
 // A workgroup walks its slice in passes of R rounds; a round covers n_waves * K
-// consecutive 64-index chunks, K per wave.  All R*K loads of a pass are issued
-// up front (after the small table loads), then the rounds are processed in
-// order, each waiting only for its own loads (the host currently always picks
-// R = 1, see lplb_map_idx):
+// consecutive 64-index chunks, K per wave.  All R*K loads of the first pass are
+// issued up front (before the small table loads are used), those of every later
+// pass while the pass before it is still being ranked and stored; the rounds are
+// then processed in order (the host currently always picks R = 1, see lplb_map_idx):
 //   A  each wave histograms its K chunks into its own LDS counter row;
 //   B  each wave turns the rows into its starting ordinals (running total of
 //      earlier slices and rounds + counts of the waves before it);
@@ -82,19 +82,28 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   const float share0 = rep0 ? a.o_weight[rank0 * a.D + local0 % a.D] : 0.0f;
   const int host0 = rep0 ? a.o2r[(rank0 % a.G) * a.D + local0 % a.D] : 0;
 
-  // Expert ids of one pass: -1 for masked / out-of-range / past the end.
+  // One pass of indices, as loaded (raw) and as expert ids (ev: -1 for masked /
+  // out-of-range / past the end).  The loads of the next pass are issued while the
+  // current one is still being ranked and stored.
+  int64_t raw[R][K];
   int32_t ev[R][K];
-  auto load_pass = [&](int64_t pass) {
+  auto issue_loads = [&](int64_t pass) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
       for (int c = 0; c < K; ++c) {
         const int64_t i = pass + r * round_len + ((int64_t)wave * K + c) * kWave + lane;
-        const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
-        ev[r][c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
+        raw[r][c] = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
       }
   };
-  load_pass(begin);
+  auto take_loads = [&]() {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        ev[r][c] = (raw[r][c] >= 0 && raw[r][c] < nl) ? (int32_t)raw[r][c] : -1;
+  };
+  issue_loads(begin);
 
   const RedirectShape sh{nl, a.n_ranks, a.G, a.D, a.C, a.L, a.P};
   if (e0 < nl)
@@ -123,8 +132,7 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
 
   int parity = 0;   // which half of counts / carry the current round uses
   for (int64_t pass = begin; pass < end; pass += R * round_len) {
-    if (pass != begin)
-      load_pass(pass);
+    take_loads();
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t round = pass + r * round_len;
@@ -135,6 +143,8 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
         for (int c = 0; c < K; ++c)
           if (ev[r][c] >= 0)
             atomicAdd(&my_counts[ev[r][c]], 1);
+        if (r == R - 1 && pass + R * round_len < end)
+          issue_loads(pass + R * round_len);   // in flight during the barrier, phases B and C
         if (r == 0) LPLB_MAP_STAMP(2);
         __syncthreads();
         if (r == 0) LPLB_MAP_STAMP(3);
@@ -248,10 +258,17 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   a.clocks = nullptr;
 #endif
 
-  // One wave per 64-index chunk of the slice, up to 16 waves, as LDS allows;
-  // then up to 8 chunks per wave and round.
+  // One wave per 64-index chunk of the slice, as LDS allows, then up to 8 chunks per
+  // wave and pass.  At most 16 waves when there is one workgroup per CU; with more
+  // workgroups than CUs smaller ones (8, then 4 waves) share a CU, and one's ranking
+  // phases overlap another's loads and stores (measured at 512 MiB in + 512 MiB out:
+  // 1024 slices of 4 waves 4.9 TB/s, 256 slices of 16 waves 4.1 TB/s).
   const int64_t chunks = (a.per + kWave - 1) / kWave;
-  int n_waves = chunks < kMaxWaves ? (int)chunks : kMaxWaves;
+  const int n_cus = current_device_cu_count();
+  int max_waves = kMaxWaves;
+  while (max_waves > 4 && n_cus > 0 && (int64_t)n_blocks * max_waves > (int64_t)kMaxWaves * n_cus)
+    max_waves >>= 1;
+  int n_waves = chunks < max_waves ? (int)chunks : max_waves;
   constexpr size_t kLdsLimit = 160 * 1024;
   while (n_waves > 1 && map_lds_bytes(a.n_logical, n_waves) > kLdsLimit)
     n_waves >>= 1;
