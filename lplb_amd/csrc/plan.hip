@@ -336,7 +336,7 @@ static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t
 // LP shapes the one-launch plan is built for, in the order they are tried, and the
 // workgroup size that leaves the LP its registers: 128 VGPRs per lane at 16 waves,
 // 256 at 8.
-constexpr int kPlanShapes[][2] = {{8, 1}, {8, 2}, {8, 4}, {16, 1}, {16, 2}};
+constexpr int kPlanShapes[][2] = {{8, 1}, {8, 2}, {8, 4}, {16, 1}, {16, 2}, {32, 1}, {32, 2}};
 constexpr int plan_waves(int gm, int dm) { return (gm * dm <= 16 && gm <= 16) ? 16 : 8; }
 static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
   for (const auto &shape : kPlanShapes)
@@ -441,6 +441,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
     err = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true>(a, s)                        \
                                : launch_plan_shape<GM, DM, false>(a, s);
   LPLB_PLAN_CASE(8, 1) LPLB_PLAN_CASE(8, 2) LPLB_PLAN_CASE(8, 4) LPLB_PLAN_CASE(16, 1) LPLB_PLAN_CASE(16, 2)
+  LPLB_PLAN_CASE(32, 1) LPLB_PLAN_CASE(32, 2)
 #undef LPLB_PLAN_CASE
   LPLB_HIP_TRY(err);
   *done = true;
