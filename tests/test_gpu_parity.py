@@ -481,19 +481,24 @@ def test_planner_run_equals_plan_with_local_counts(cuda):
     assert torch.equal(got, want) and int(a1[0]) == int(a2[0]) == 1
 
 
-def test_plan_replays_from_a_hip_graph(cuda):
+@pytest.mark.parametrize("use_global", [True, False])
+def test_plan_replays_from_a_hip_graph(cuda, use_global):
     """Capture two plans into a graph; every replay, with eager work and synchronisation between
-    replays, must reproduce the eager result and advance the counter."""
+    replays, must reproduce the eager result and advance the counter.  (The one-launch plan keeps
+    counters in device memory that its last workgroup clears: a replay has the same arguments.)"""
     inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    counts = t["counts"] if use_global else None
     avail = torch.zeros(1, dtype=torch.int32, device=cuda)
-    eager, eager_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])
+    eager, eager_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts)
     torch.cuda.synchronize()
     ws = {"out": torch.empty_like(eager), "o_weight": torch.empty_like(eager_w),
           "by_sm": torch.empty(256, shape.n_logical, dtype=torch.int32, device=cuda),
           "global_workload": torch.empty(shape.n_logical, dtype=torch.float32, device=cuda)}
+    phys = torch.empty(shape.n_physical, dtype=torch.int32, device=cuda)
 
     def plan():
-        solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"], workspace=ws)
+        solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts, workspace=ws,
+                    physical_counts=phys)
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -509,13 +514,40 @@ def test_plan_replays_from_a_hip_graph(cuda):
     for rep in range(4):
         ws["out"].fill_(-5)
         ws["o_weight"].zero_()
+        phys.fill_(-5)
         scratch = torch.randn(1 << 16, device=cuda).sum()      # unrelated eager work between replays
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(ws["out"], eager) and torch.equal(ws["o_weight"], eager_w), rep
         assert int(avail[0]) == before + 2 * (rep + 1)
+        assert torch.equal(phys.long(), torch.bincount(eager[eager >= 0].flatten(), minlength=shape.n_physical))
         del scratch
+
+
+def test_plans_on_two_streams_with_the_chain(cuda):
+    """Plans that may overlap on one device (two streams) must use the chain of kernels
+    (`set_plan_cooperative(False)`): the one-launch form keeps per-device counters."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    other = synth.make_inputs("v3_ep8_cube", tokens=5000, mask_fraction=0.1)
+    idx_b = dev(other.indices, cuda)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want_a, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)
+    want_b, _, _ = solver.plan(idx_b, t["r2o"], t["o2r"], t["phy2log"], avail, 256)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    _native.set_plan_cooperative(False)
+    try:
+        for rep in range(20):
+            outs = []
+            for s_, idx in zip(streams, (t["idx"], idx_b)):
+                with torch.cuda.stream(s_):
+                    outs.append(solver.plan(idx, t["r2o"], t["o2r"], t["phy2log"], avail, 256)[0])
+            torch.cuda.synchronize()
+            assert torch.equal(outs[0], want_a) and torch.equal(outs[1], want_b), rep
+    finally:
+        _native.set_plan_cooperative(True)
 
 
 def test_kernel_timestamp_hook(cuda):
