@@ -180,8 +180,11 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  *   out              int64 [n_elements], out (see lplb_map_idx)
  *   physical_counts  int32 [n_physical] or NULL, out (see lplb_map_idx)
  *
- * The one-launch form keeps three counters in a per-device array of the library:
- * plans of one device must be enqueued on one stream (or otherwise not overlap).
+ * The one-launch form keeps its counters in a per-device array of the library, one
+ * block for each of the first two streams that plan (further streams get the
+ * chain).  Launches that share a block must not overlap in time, which stream order
+ * guarantees; the exception is a graph captured on one stream and replayed
+ * concurrently on several (see lplb_plan_set_cooperative).
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -194,9 +197,10 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
 
 /*
  * No counterpart in the reference.  enabled = 0 makes lplb_plan always run the
- * chain of kernels (for callers that overlap plans of one device on several
- * streams, or that fill the GPU with other resident kernels); 1 (the default)
- * lets it use the one-launch form where that applies.  Process-wide.
+ * chain of kernels (for callers that replay captured plans concurrently on
+ * several streams, or that keep the GPU full of kernels which themselves wait for
+ * a plan); 1 (the default) lets it use the one-launch form where that applies.
+ * Process-wide.
  */
 int lplb_plan_set_cooperative(int enabled);
 

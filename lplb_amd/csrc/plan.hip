@@ -26,12 +26,15 @@
 // than the GPU (at most 65 workgroups on 256 CUs), so all workgroups are resident
 // and the waits end; each wait is bounded all the same, and a wait that runs out is
 // counted (lplb_plan_sync_timeouts) instead of hanging the GPU.  The counters live
-// in a per-device array of this library; the last workgroup to leave clears them.
-// Launches of this kernel that overlap on one device (different streams) would
-// share them: run plans of one device on one stream, or switch this path off with
-// lplb_plan_set_cooperative(0).
+// in a per-device array of this library, one block per stream (the first two streams
+// that run a plan; further streams get the chain); the last workgroup to leave
+// clears its block, so a captured launch can be replayed.  Launches that share a
+// block must not overlap in time: that holds for one stream's launches, not for
+// graphs captured on one stream and replayed concurrently on several -- such
+// callers switch this path off with lplb_plan_set_cooperative(0).
 #include "map_kernel.h"
 #include "solve_kernel.h"
+#include <mutex>
 
 namespace lplb {
 
@@ -47,7 +50,12 @@ constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait 
 // which every slice adds its row.
 constexpr int kSharesAt = 16, kMaxShares = 256;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
-static __device__ __attribute__((aligned(64))) int g_plan_sync[kTotalsAt + kMaxTotals];
+// One such block per stream that has run a plan, so that plans enqueued on different
+// streams do not share counters.  Two blocks, because a launch takes at most half of
+// the CUs: two launches are then still resident together, more might not be (and
+// workgroups that wait for workgroups that cannot start would wait for ever).
+constexpr int kSlotInts = kTotalsAt + kMaxTotals, kSyncSlots = 2;
+static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
 static bool g_cooperative = true;
 
 struct PlanArgs {
@@ -364,6 +372,23 @@ template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanAr
   return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s);
 }
 
+// The block of counters a stream uses: the first kSyncSlots streams that run a plan
+// each get their own, -1 for any further one (which then runs the chain).  The null
+// stream and a torch side stream are the usual two.
+static int sync_slot_of(hipStream_t s) {
+  static std::mutex guard;
+  static hipStream_t owner[kSyncSlots];
+  static int used = 0;
+  std::lock_guard<std::mutex> lock(guard);
+  for (int i = 0; i < used; ++i)
+    if (owner[i] == s)
+      return i;
+  if (used == kSyncSlots)
+    return -1;
+  owner[used] = s;
+  return used++;
+}
+
 // Per-device address of the counters and CU count, looked up once.
 static int plan_device_state(int **sync, int *n_cus) {
   static int *sync_of[64];
@@ -417,8 +442,10 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   int rc = plan_device_state(&sync, &n_cus);
   if (rc != LPLB_OK)
     return rc;
-  if (slices + 1 > n_cus / 2)
+  const int slot = sync_slot_of(s);
+  if (slices + 1 > n_cus / 2 || slot < 0)
     return LPLB_OK;
+  sync += (size_t)slot * kSlotInts;
 
   PlanArgs a{};   // every field the host does not set below is zero
   a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices;
@@ -462,7 +489,12 @@ extern "C" int lplb_plan_sync_timeouts(int *count) {
   int rc = plan_device_state(&sync, &n_cus);
   if (rc != LPLB_OK)
     return rc;
-  LPLB_HIP_TRY(hipMemcpy(count, sync + 3, sizeof(int), hipMemcpyDeviceToHost));
+  *count = 0;
+  for (int slot = 0; slot < kSyncSlots; ++slot) {
+    int n = 0;
+    LPLB_HIP_TRY(hipMemcpy(&n, sync + (size_t)slot * kSlotInts + 3, sizeof(int), hipMemcpyDeviceToHost));
+    *count += n;
+  }
   return LPLB_OK;
 }
 

@@ -525,9 +525,11 @@ def test_plan_replays_from_a_hip_graph(cuda, use_global):
         del scratch
 
 
-def test_plans_on_two_streams_with_the_chain(cuda):
-    """Plans that may overlap on one device (two streams) must use the chain of kernels
-    (`set_plan_cooperative(False)`): the one-launch form keeps per-device counters."""
+@pytest.mark.parametrize("cooperative", [False, True])
+def test_plans_on_two_streams(cuda, cooperative):
+    """Plans on different streams may overlap on the device.  The one-launch form keeps its
+    counters per stream (for the first two streams that plan; later ones get the chain), and the
+    chain of kernels has no shared state at all."""
     from lplb_amd import _native
     inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
     other = synth.make_inputs("v3_ep8_cube", tokens=5000, mask_fraction=0.1)
@@ -536,16 +538,17 @@ def test_plans_on_two_streams_with_the_chain(cuda):
     want_a, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)
     want_b, _, _ = solver.plan(idx_b, t["r2o"], t["o2r"], t["phy2log"], avail, 256)
     torch.cuda.synchronize()
-    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
-    _native.set_plan_cooperative(False)
+    streams = [torch.cuda.current_stream(), torch.cuda.Stream(), torch.cuda.Stream()]
+    _native.set_plan_cooperative(cooperative)
     try:
-        for rep in range(20):
+        for rep in range(30):
             outs = []
-            for s_, idx in zip(streams, (t["idx"], idx_b)):
+            for s_, idx in zip(streams, (t["idx"], idx_b, t["idx"])):
                 with torch.cuda.stream(s_):
                     outs.append(solver.plan(idx, t["r2o"], t["o2r"], t["phy2log"], avail, 256)[0])
             torch.cuda.synchronize()
-            assert torch.equal(outs[0], want_a) and torch.equal(outs[1], want_b), rep
+            assert torch.equal(outs[0], want_a) and torch.equal(outs[1], want_b) and torch.equal(outs[2], want_a), rep
+        assert _native.plan_sync_timeouts() == 0
     finally:
         _native.set_plan_cooperative(True)
 
