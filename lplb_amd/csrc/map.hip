@@ -6,19 +6,18 @@
 // from a shared-memory atomic (minilp.cu:504), which fixes the set of ordinals
 // per block but not which token gets which.  Here k is canonical.
 //
-// A workgroup walks its slice in passes of R rounds; a round covers n_waves * K
-// consecutive 64-index chunks, K per wave.  All R*K loads of the first pass are
-// issued up front (before the small table loads are used), those of every later
-// pass while the pass before it is still being ranked and stored; the rounds are
-// then processed in order (the host currently always picks R = 1, see lplb_map_idx):
+// A workgroup walks its slice in passes of n_waves * K consecutive 64-index chunks,
+// K per wave.  The loads of the first pass are issued up front (before the small
+// table loads are used), those of every later pass while the pass before it is
+// still being ranked and stored.  Per pass:
 //   A  each wave histograms its K chunks into its own LDS counter row;
 //   B  each wave turns the rows into its starting ordinals (running total of
-//      earlier slices and rounds + counts of the waves before it);
+//      earlier slices and passes + counts of the waves before it);
 //   C  chunk by chunk, lanes holding the same expert find each other through a
 //      per-wave 64-bit LDS bitmap (one OR, one 16-byte read); the rank among those
 //      peers is a popcount of lower lanes and the last peer advances the counter.
-// Counter rows and running totals are double-buffered by round parity, which
-// leaves one workgroup barrier per round.  Nothing depends on execution order.
+// Counter rows and running totals are double-buffered by pass parity, which
+// leaves one workgroup barrier per pass.  Nothing depends on execution order.
 // The modulo of the hash uses a per-expert reciprocal prepared with the tables.
 #include "map_kernel.h"
 
@@ -46,7 +45,7 @@ __global__ void zero_ints(int32_t *p, int n) {
     p[i] = 0;
 }
 
-template <int K, int R, bool WRAP>
+template <int K, bool WRAP>
 __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int nl = a.n_logical;
@@ -63,7 +62,7 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
 
   const int64_t begin = slice_begin(a.n, a.per, pid);
   const int64_t end = slice_begin(a.n, a.per, pid + 1);
-  const int64_t round_len = (int64_t)n_waves * K * kWave;
+  const int64_t pass_len = (int64_t)n_waves * K * kWave;
   WaveSlot *mine = slots + (size_t)wave * nl;
   const unsigned long long my_bit = 1ull << lane;
   LPLB_MAP_STAMP(0);
@@ -85,23 +84,19 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   // One pass of indices, as loaded (raw) and as expert ids (ev: -1 for masked /
   // out-of-range / past the end).  The loads of the next pass are issued while the
   // current one is still being ranked and stored.
-  int64_t raw[R][K];
-  int32_t ev[R][K];
+  int64_t raw[K];
+  int32_t ev[K];
   auto issue_loads = [&](int64_t pass) {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int c = 0; c < K; ++c) {
-        const int64_t i = pass + r * round_len + ((int64_t)wave * K + c) * kWave + lane;
-        raw[r][c] = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
-      }
+    for (int c = 0; c < K; ++c) {
+      const int64_t i = pass + ((int64_t)wave * K + c) * kWave + lane;
+      raw[c] = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
+    }
   };
   auto take_loads = [&]() {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int c = 0; c < K; ++c)
-        ev[r][c] = (raw[r][c] >= 0 && raw[r][c] < nl) ? (int32_t)raw[r][c] : -1;
+    for (int c = 0; c < K; ++c)
+      ev[c] = (raw[c] >= 0 && raw[c] < nl) ? (int32_t)raw[c] : -1;
   };
   issue_loads(begin);
 
@@ -130,61 +125,55 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   // (the barrier after the first phase A also publishes the tables)
   LPLB_MAP_STAMP(1);
 
-  int parity = 0;   // which half of counts / carry the current round uses
-  for (int64_t pass = begin; pass < end; pass += R * round_len) {
+  int parity = 0;   // which half of counts / carry the current pass uses
+  for (int64_t pass = begin; pass < end; pass += pass_len) {
     take_loads();
+    int32_t *my_counts = counts + ((size_t)parity * n_waves + wave) * nl;
+    // Phase A: tokens per expert in this wave's chunks.
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t round = pass + r * round_len;
-      if (round < end) {   // uniform over the workgroup
-        int32_t *my_counts = counts + ((size_t)parity * n_waves + wave) * nl;
-        // Phase A: tokens per expert in this wave's chunks.
+    for (int c = 0; c < K; ++c)
+      if (ev[c] >= 0)
+        atomicAdd(&my_counts[ev[c]], 1);
+    if (pass + pass_len < end)
+      issue_loads(pass + pass_len);   // in flight during the barrier, phases B and C
+    LPLB_MAP_STAMP(2);
+    __syncthreads();
+    LPLB_MAP_STAMP(3);
+    // Phase B: every wave derives its own starting ordinals: the running total
+    // of earlier slices and passes plus the counts of the waves before it.  The
+    // last wave writes the next pass's running total into the other half, and
+    // every wave clears its row of the other half for the next pass.
+    const int32_t *pass_counts = counts + (size_t)parity * n_waves * nl;
+    int32_t *other_counts = counts + ((size_t)(parity ^ 1) * n_waves + wave) * nl;
+    for (int e = lane; e < nl; e += kWave) {
+      // all reads in flight before the first add
+      int32_t before[kMaxWaves];
 #pragma unroll
-        for (int c = 0; c < K; ++c)
-          if (ev[r][c] >= 0)
-            atomicAdd(&my_counts[ev[r][c]], 1);
-        if (r == R - 1 && pass + R * round_len < end)
-          issue_loads(pass + R * round_len);   // in flight during the barrier, phases B and C
-        if (r == 0) LPLB_MAP_STAMP(2);
-        __syncthreads();
-        if (r == 0) LPLB_MAP_STAMP(3);
-        // Phase B: every wave derives its own starting ordinals: the running total
-        // of earlier slices and rounds plus the counts of the waves before it.  The
-        // last wave writes the next round's running total into the other half, and
-        // every wave clears its row of the other half for the next round.
-        const int32_t *round_counts = counts + (size_t)parity * n_waves * nl;
-        int32_t *other_counts = counts + ((size_t)(parity ^ 1) * n_waves + wave) * nl;
-        for (int e = lane; e < nl; e += kWave) {
-          // all reads in flight before the first add
-          int32_t before[kMaxWaves];
+      for (int w = 0; w < kMaxWaves; ++w)
+        before[w] = w < wave ? pass_counts[(size_t)w * nl + e] : 0;
+      int32_t run = carry[parity * nl + e];
+      const int32_t own = my_counts[e];
 #pragma unroll
-          for (int w = 0; w < kMaxWaves; ++w)
-            before[w] = w < wave ? round_counts[(size_t)w * nl + e] : 0;
-          int32_t run = carry[parity * nl + e];
-          const int32_t own = my_counts[e];
-#pragma unroll
-          for (int w = 0; w < kMaxWaves; ++w)
-            run += before[w];
-          mine[e].next = run;
-          if (wave == n_waves - 1)
-            carry[(parity ^ 1) * nl + e] = run + own;
-          other_counts[e] = 0;
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (r == 0) LPLB_MAP_STAMP(4);
-        // Phase C.
-#pragma unroll
-        for (int c = 0; c < K; ++c) {
-          const int64_t o = redirect_token<WRAP>(ev[r][c], mine, table, replica, my_bit);
-          const int64_t i = round + ((int64_t)wave * K + c) * kWave + lane;
-          if (i < end)
-            __builtin_nontemporal_store(o, a.out + i);
-          __builtin_amdgcn_wave_barrier();
-        }
-        if (r == 0) LPLB_MAP_STAMP(5);
-        parity ^= 1;
-      }
+      for (int w = 0; w < kMaxWaves; ++w)
+        run += before[w];
+      mine[e].next = run;
+      if (wave == n_waves - 1)
+        carry[(parity ^ 1) * nl + e] = run + own;
+      other_counts[e] = 0;
     }
+    __builtin_amdgcn_wave_barrier();
+    LPLB_MAP_STAMP(4);
+    // Phase C.
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const int64_t o = redirect_token<WRAP>(ev[c], mine, table, replica, my_bit);
+      const int64_t i = pass + ((int64_t)wave * K + c) * kWave + lane;
+      if (i < end)
+        __builtin_nontemporal_store(o, a.out + i);
+      __builtin_amdgcn_wave_barrier();
+    }
+    LPLB_MAP_STAMP(5);
+    parity ^= 1;
   }
   if (pid == 0 && a.physical_counts)   // the tables are complete since the first barrier
     emit_physical_counts(table, replica, sh, a.phy2log, a.physical_counts, tid, nt);
@@ -197,16 +186,16 @@ static size_t map_lds_bytes(int n_logical, int w) {
   return (size_t)n_logical * (sizeof(ExpertEntry) + 4 + 8 + (size_t)w * (sizeof(WaveSlot) + 8));
 }
 
-template <int K, int R, bool WRAP>
+template <int K, bool WRAP>
 static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
   if (lds > 64 * 1024) {
     // above the default limit the kernel has to be told once per process
-    static hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&redirect_indices<K, R, WRAP>),
+    static hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&redirect_indices<K, WRAP>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (raised != hipSuccess)
       return raised;
   }
-  launch(redirect_indices<K, R, WRAP>, grid, block, lds, s, a);
+  launch(redirect_indices<K, WRAP>, grid, block, lds, s, a);
   return hipGetLastError();
 }
 
@@ -278,21 +267,21 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   const size_t lds = map_lds_bytes(a.n_logical, n_waves);
   const dim3 grid(n_blocks), block(n_waves * kWave);
   hipError_t err;
-#define LPLB_MAP_CASE(K, R)                                                                    \
-  err = wrap ? launch_redirect<K, R, true>(a, grid, block, lds, s)                             \
-             : launch_redirect<K, R, false>(a, grid, block, lds, s)
-  // K chunks per wave and round, R rounds per pass (K * R loads in flight per
-  // lane).  Measured at [262144 x 8] on MI355X: a round costs about 2.5 us of
-  // barrier skew and counter traffic, more than splitting a pass into rounds can
-  // hide, so a pass is one round of up to 8 chunks; longer slices loop over passes.
+#define LPLB_MAP_CASE(K)                                                                    \
+  err = wrap ? launch_redirect<K, true>(a, grid, block, lds, s)                             \
+             : launch_redirect<K, false>(a, grid, block, lds, s)
+  // K chunks per wave and pass (K loads in flight per lane, K more prefetched).
+  // Measured at [262144 x 8] on MI355X: a pass costs about 2.5 us of barrier skew
+  // and counter traffic, so a pass is as long as registers allow (8 chunks per
+  // wave); longer slices loop over passes.
   if (per_wave <= 1) {
-    LPLB_MAP_CASE(1, 1);
+    LPLB_MAP_CASE(1);
   } else if (per_wave <= 2) {
-    LPLB_MAP_CASE(2, 1);
+    LPLB_MAP_CASE(2);
   } else if (per_wave <= 4) {
-    LPLB_MAP_CASE(4, 1);
+    LPLB_MAP_CASE(4);
   } else {
-    LPLB_MAP_CASE(8, 1);
+    LPLB_MAP_CASE(8);
   }
 #undef LPLB_MAP_CASE
   LPLB_HIP_TRY(err);
