@@ -9,8 +9,9 @@
 // as a parallel branch of a captured HIP graph (side stream + events) was measured
 // and rejected: 24.6 us per plan against 20.0 us for the plain chain in the graph.
 //
-// One launch (plan_in_one_launch): for batches of up to 64 slices of 2048 indices
-// and LP shapes whose registers fit beside a 512- or 1024-thread workgroup.  Every
+// One launch (plan_in_one_launch): for batches of up to 64 slices of 4096 indices
+// (2048 with 512-thread workgroups) and LP shapes whose registers fit beside a 512-
+// or 1024-thread workgroup.  Every
 // kernel boundary of the chain costs 3-5 us on this GPU although the kernels have
 // 1-3 us of work, and the LP (8 us, one wave) sits on the critical path.  Here one
 // workgroup per slice and one more for the LP run side by side in a single grid:
@@ -38,8 +39,8 @@
 
 namespace lplb {
 
-constexpr int kSliceIndices = 2048;   // longest slice of the one-launch plan
-constexpr int kMaxSlices = 64;
+constexpr int kMaxSlices = 64;         // slice workgroups of the one-launch plan
+constexpr int kChunksPerWave = 4;     // its longest slice: 4 chunks of 64 indices per wave
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
 constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait gives up
 
@@ -416,7 +417,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   *done = false;
   const int L = P - D * C, n_fixed = L - D * C;
   const int n_logical = n_group * G * L;
-  if (!g_cooperative || n_elements <= 0 || n_elements > (int64_t)kMaxSlices * kSliceIndices || n_blocks < 2)
+  if (!g_cooperative || n_elements <= 0 || n_blocks < 2)
     return LPLB_OK;
   int gm = 0, dm = 0;
   if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || n_group * G * D > kMaxShares || global_workload == nullptr)
@@ -425,18 +426,18 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   // own-histogram mode: a spare wave beside the LPs, the totals fit the accumulator and the LDS
   if (counts == nullptr && (n_group >= waves || n_logical > kMaxTotals))
     return LPLB_OK;
-  // slices of 1024 indices while 64 of them cover the batch, at most n_blocks - 1
-  // (the caller's bound on parallelism; the last row of its table takes the totals)
-#ifndef LPLB_PLAN_FIRST_SLICE
-#define LPLB_PLAN_FIRST_SLICE 1024
-#endif
-  int64_t slices = (n_elements + LPLB_PLAN_FIRST_SLICE - 1) / LPLB_PLAN_FIRST_SLICE;
+  // slices of 1024 indices while kMaxSlices of them cover the batch, else of 2048, else of
+  // 4096; at most n_blocks - 1 of them (the caller's bound on parallelism; the last row of
+  // its table takes the totals)
+  int64_t slices = kMaxSlices + 1;
+  for (int64_t len = 1024; len <= (int64_t)waves * kChunksPerWave * kWave && slices > kMaxSlices; len *= 2)
+    slices = (n_elements + len - 1) / len;
   if (slices > kMaxSlices)
-    slices = (n_elements + kSliceIndices - 1) / kSliceIndices;
+    return LPLB_OK;
   if (slices > n_blocks - 1)
     slices = n_blocks - 1;
   const int64_t per = slice_len(n_elements, (int)slices);
-  if (per > (int64_t)waves * 4 * kWave || plan_lds_bytes(n_logical, waves) > (size_t)kPlanLdsLimit)
+  if (per > (int64_t)waves * kChunksPerWave * kWave || plan_lds_bytes(n_logical, waves) > (size_t)kPlanLdsLimit)
     return LPLB_OK;
   int *sync = nullptr, n_cus = 0;
   int rc = plan_device_state(&sync, &n_cus);

@@ -433,7 +433,7 @@ def test_plan_entry_point_matches_three_calls(cuda, cfg, use_global):
 
 @pytest.mark.parametrize("cfg", ["cpu_ref_ep8", "v3_ep8_cube", "ep16_hypercube", "ep32_torus"])
 @pytest.mark.parametrize("use_global", [True, False])
-@pytest.mark.parametrize("tokens,n_sms", [(None, 256), (37, 256), (4100, 9), (16384, 40), (20000, 256)])
+@pytest.mark.parametrize("tokens,n_sms", [(None, 256), (37, 256), (4100, 9), (16384, 40), (20000, 256), (32768, 65), (40000, 256)])
 def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
     """Short batches run as one kernel launch whose workgroups exchange histogram rows and the
     LP's shares through memory; the result must be the chain's, bit for bit, call after call."""
