@@ -161,7 +161,12 @@ class Planner:
             out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
                                                       physical_counts=physical_counts)
             return out
-        local_workload, local_workload_by_sm = self.count_workload(idx, n_sms)
-        o_weight, _global_workload = self.solve_probs(local_workload, avail_counter)
-        return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256,
-                                   physical_counts=physical_counts)
+        # With a process group the counts have to be summed over the ranks between histogram and
+        # LP (lplb/planner.py:214-216); LP and redirect then run as one plan on the summed counts.
+        local_workload, _by_sm = self.count_workload(idx, n_sms)
+        workload = local_workload.clone()
+        if not self.deep_ep_initialized:
+            torch.distributed.all_reduce(workload, group=self.ep_group)
+        out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
+                                                  global_counts=workload, physical_counts=physical_counts)
+        return out

@@ -481,6 +481,36 @@ def test_planner_run_equals_plan_with_local_counts(cuda):
     assert torch.equal(got, want) and int(a1[0]) == int(a2[0]) == 1
 
 
+def test_planner_run_with_a_process_group(cuda, monkeypatch):
+    """With a group, run() sums the local histogram over the ranks before the LP (lplb/planner.py:214-216).
+    The collective is stubbed here (one GPU): it adds what the other ranks would contribute."""
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    c = inp.cfg
+    local = np.bincount(inp.indices[inp.indices >= 0].ravel(), minlength=c.n_logical).astype(np.int32)
+    others = dev(inp.global_counts - np.minimum(local, inp.global_counts), cuda)
+    calls = []
+
+    def fake_all_reduce(tensor, group=None):
+        calls.append(group)
+        tensor += others.view_as(tensor)
+
+    monkeypatch.setattr(torch.distributed, "all_reduce", fake_all_reduce)
+    group = object()
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size, group)
+    planner.phy2log = t["phy2log"]
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    out = planner.run(t["idx"], avail, 256)
+    assert calls == [group] and int(avail[0]) == shape.n_group
+    summed = dev(local, cuda) + others
+    avail2 = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail2, 256, global_counts=summed)
+    assert torch.equal(out, want)
+    # the three public steps give the same (lplb/planner.py:264-266)
+    lw, by_sm = planner.count_workload(t["idx"], 256)
+    o_weight, _ = planner.solve_probs(lw, avail2)
+    assert torch.equal(planner.weighted_select_target(t["idx"], o_weight, by_sm, 256), out)
+
+
 @pytest.mark.parametrize("use_global", [True, False])
 def test_plan_replays_from_a_hip_graph(cuda, use_global):
     """Capture two plans into a graph; every replay, with eager work and synchronisation between
