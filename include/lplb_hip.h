@@ -181,10 +181,12 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  *   physical_counts  int32 [n_physical] or NULL, out (see lplb_map_idx)
  *
  * The one-launch form keeps its counters in a per-device array of the library, one
- * block for each of the first two streams that plan (further streams get the
+ * block for each of the first eight streams that plan (further streams get the
  * chain).  Launches that share a block must not overlap in time, which stream order
  * guarantees; the exception is a graph captured on one stream and replayed
- * concurrently on several (see lplb_plan_set_cooperative).
+ * concurrently on several.  A launch takes up to a quarter of the GPU's CUs and its
+ * workgroups wait for each other, so at most three plans may execute at the same
+ * time on a device (see lplb_plan_set_cooperative).
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -198,8 +200,8 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
 /*
  * No counterpart in the reference.  enabled = 0 makes lplb_plan always run the
  * chain of kernels (for callers that replay captured plans concurrently on
- * several streams, or that keep the GPU full of kernels which themselves wait for
- * a plan); 1 (the default) lets it use the one-launch form where that applies.
+ * several streams, that let four or more plans execute at once, or that keep the
+ * GPU full of kernels which themselves wait for a plan); 1 (the default) lets it use the one-launch form where that applies.
  * Process-wide.
  */
 int lplb_plan_set_cooperative(int enabled);

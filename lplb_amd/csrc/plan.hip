@@ -27,12 +27,13 @@
 // than the GPU (at most 65 workgroups on 256 CUs), so all workgroups are resident
 // and the waits end; each wait is bounded all the same, and a wait that runs out is
 // counted (lplb_plan_sync_timeouts) instead of hanging the GPU.  The counters live
-// in a per-device array of this library, one block per stream (the first two streams
+// in a per-device array of this library, one block per stream (the first eight streams
 // that run a plan; further streams get the chain); the last workgroup to leave
 // clears its block, so a captured launch can be replayed.  Launches that share a
 // block must not overlap in time: that holds for one stream's launches, not for
-// graphs captured on one stream and replayed concurrently on several -- such
-// callers switch this path off with lplb_plan_set_cooperative(0).
+// graphs captured on one stream and replayed concurrently on several; and no more
+// than three plans may execute at the same time on a device -- callers outside
+// these limits switch this path off with lplb_plan_set_cooperative(0).
 #include "map_kernel.h"
 #include "solve_kernel.h"
 #include <mutex>
@@ -51,11 +52,12 @@ constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait 
 // which every slice adds its row.
 constexpr int kSharesAt = 16, kMaxShares = 256;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
-// One such block per stream that has run a plan, so that plans enqueued on different
-// streams do not share counters.  Two blocks, because a launch takes at most half of
-// the CUs: two launches are then still resident together, more might not be (and
-// workgroups that wait for workgroups that cannot start would wait for ever).
-constexpr int kSlotInts = kTotalsAt + kMaxTotals, kSyncSlots = 2;
+// One such block per stream that has run a plan (the compute stream, a warm-up
+// stream, a graph-capture stream ...), so that plans enqueued on different streams
+// do not share counters.  A launch takes at most a quarter of the CUs: up to three
+// plans that really execute at the same time are all resident; with four or more,
+// workgroups could wait for workgroups that cannot start.
+constexpr int kSlotInts = kTotalsAt + kMaxTotals, kSyncSlots = 8;
 static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
 static bool g_cooperative = true;
 
@@ -374,8 +376,7 @@ template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanAr
 }
 
 // The block of counters a stream uses: the first kSyncSlots streams that run a plan
-// each get their own, -1 for any further one (which then runs the chain).  The null
-// stream and a torch side stream are the usual two.
+// each get their own, -1 for any further one (which then runs the chain).
 static int sync_slot_of(hipStream_t s) {
   static std::mutex guard;
   static hipStream_t owner[kSyncSlots];
@@ -444,7 +445,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (rc != LPLB_OK)
     return rc;
   const int slot = sync_slot_of(s);
-  if (slices + 1 > n_cus / 2 || slot < 0)
+  if (slices + 1 > n_cus / 4 + 1 || slot < 0)
     return LPLB_OK;
   sync += (size_t)slot * kSlotInts;
 
