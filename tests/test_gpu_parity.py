@@ -147,6 +147,46 @@ def test_physical_counts_when_499_divides_a_total(cuda, multiple):
         np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
 
 
+def test_count_and_redirect_random_shapes(cuda):
+    """Forty seeded draws of batch length, slice count, topology and weights: histogram table and
+    redirected indices bit-exact against the oracle, counts per physical expert against its bincount."""
+    from lplb_amd import topology
+    from lplb_amd.mapping import build_redundancy_mapping
+    rng = np.random.default_rng(2024)
+    topologies = [(topology.CUBE_8P2E, 1), (topology.RING_8P, 1), (topology.HYPERCUBE_16P2E, 1),
+                  (topology.torus_2d(8, 4), 1), (topology.CUBE_8P2E, 4), (_shifted_ring(6, [1, 2]), 2),
+                  (_shifted_ring(4, [1, 2, 3]), 3)]
+    for trial in range(40):
+        r2o, n_group = topologies[int(rng.integers(len(topologies)))]
+        r2o = np.asarray(r2o, np.int32)
+        g, d = r2o.shape
+        ep = g * n_group
+        combined = int(rng.integers(1, 3))
+        per_rank = d * combined + int(rng.integers(d * combined, 12))       # at least as many as replicas
+        n_logical = ep * per_rank
+        shape = Shape(r2o, ep, n_logical, n_logical + d * combined * ep)
+        hist = rng.integers(1, 1 << 20, size=n_logical).astype(np.int64)
+        phy2log, _, _ = build_redundancy_mapping(r2o, ep, n_logical, shape.n_physical, hist, n_nodes=1)
+        n = int(rng.choice([0, 1, 63, 64, 65, 255, 256, 257, 1000, 4097, 70000, 300001]))
+        n_sms = int(rng.choice([1, 2, 3, 17, 64, 255, 256, 304, 700]))
+        idx = rng.integers(-1, n_logical, size=n, dtype=np.int64)
+        if n and trial % 5 == 0:
+            idx[rng.integers(0, n, size=max(1, n // 50))] = n_logical + int(rng.integers(0, 5))   # out of range
+        o_weight = _random_weights(shape, rng)
+        solver = solver_for(shape)
+        d_idx = dev(idx, cuda)
+        total, by_sm = solver.count_idx(d_idx, n_sms)
+        want_by = oracle.count_idx(idx, n_logical, n_sms)
+        np.testing.assert_array_equal(by_sm.cpu().numpy(), want_by, err_msg=f"trial {trial}")
+        phys = torch.full((shape.n_physical,), -3, dtype=torch.int32, device=cuda)
+        got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms,
+                             physical_counts=phys).cpu().numpy()
+        want = oracle.map_idx(idx, o_weight, want_by, shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+        np.testing.assert_array_equal(got, want, err_msg=f"trial {trial}")
+        np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical),
+                                      err_msg=f"trial {trial}")
+
+
 # -------------------------------------------------------------------- solver
 def _compare_solve(shape, phy2log, workload, res, gw, avail, step_rule=0, n_steps=5):
     o_res, o_gw, o_avail = oracle.solve(workload, shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed,
@@ -467,6 +507,53 @@ def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
                                                              minlength=c.n_logical))
     out = runs[True][0]
     np.testing.assert_array_equal(runs[True][4], np.bincount(out[out >= 0].ravel(), minlength=c.n_physical))
+
+
+def test_plan_random_shapes_one_launch_equals_chain(cuda):
+    """Thirty seeded draws of topology, experts per rank, batch length and slice bound, in both LP
+    feeding modes: the one-launch plan (where it applies) and the chain agree bit for bit."""
+    from lplb_amd import _native, topology
+    from lplb_amd.mapping import build_redundancy_mapping
+    rng = np.random.default_rng(77)
+    topologies = [(topology.CUBE_8P2E, 1), (topology.RING_8P, 1), (topology.HYPERCUBE_16P2E, 1),
+                  (topology.torus_2d(8, 4), 1), (topology.CUBE_8P2E, 4), (_shifted_ring(6, [1, 2]), 2),
+                  (_shifted_ring(4, [1, 2, 3]), 3), (_shifted_ring(16, [1]), 2)]
+    try:
+        for trial in range(30):
+            r2o, n_group = topologies[int(rng.integers(len(topologies)))]
+            r2o = np.asarray(r2o, np.int32)
+            g, d = r2o.shape
+            ep = g * n_group
+            per_rank = d + int(rng.integers(d, 10))
+            n_logical = ep * per_rank
+            shape = Shape(r2o, ep, n_logical, n_logical + d * ep)
+            hist = rng.integers(1, 1 << 20, size=n_logical).astype(np.int64)
+            phy2log, _, _ = build_redundancy_mapping(r2o, ep, n_logical, shape.n_physical, hist, n_nodes=1)
+            n = int(rng.choice([1, 300, 1024, 5000, 65536, 100000, 262144, 270000]))
+            n_sms = int(rng.choice([2, 9, 64, 65, 256]))
+            popularity = rng.dirichlet(np.full(n_logical, 0.7))
+            idx = rng.choice(n_logical, size=n, p=popularity).astype(np.int64)
+            idx[rng.random(n) < 0.03] = -1
+            counts = (np.bincount(idx[idx >= 0], minlength=n_logical) * ep +
+                      rng.integers(0, 50, size=n_logical)).astype(np.int32)
+            solver = solver_for(shape)
+            t = dict(idx=dev(idx, cuda), r2o=dev(r2o, cuda), o2r=dev(shape.o2r, cuda), phy2log=dev(phy2log, cuda))
+            for global_counts in (dev(counts, cuda), None):
+                got = {}
+                for mode in (False, True):
+                    _native.set_plan_cooperative(mode)
+                    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+                    phys = torch.empty(shape.n_physical, dtype=torch.int32, device=cuda)
+                    out, w, by = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, n_sms,
+                                             global_counts=global_counts, physical_counts=phys)
+                    torch.cuda.synchronize()
+                    got[mode] = (out.cpu().numpy(), w.cpu().numpy(), by[-1].cpu().numpy(), int(avail[0]),
+                                 phys.cpu().numpy())
+                for a, b in zip(got[True], got[False]):
+                    np.testing.assert_array_equal(a, b, err_msg=f"trial {trial} {r2o.shape} n={n} n_sms={n_sms}")
+    finally:
+        _native.set_plan_cooperative(True)
+    assert _native.plan_sync_timeouts() == 0
 
 
 def test_planner_run_equals_plan_with_local_counts(cuda):
