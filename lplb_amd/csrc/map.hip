@@ -51,6 +51,7 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
   const int nl = a.n_logical;
   const int tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid % kWave, wave = tid / kWave, n_waves = nt / kWave;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, but known to be wave-uniform
   const int pid = blockIdx.x;
   ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);                 // [nl]
   WaveSlot *slots = reinterpret_cast<WaveSlot *>(table + nl);                    // [n_waves][nl]
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
       int32_t before[kMaxWaves];
 #pragma unroll
       for (int w = 0; w < kMaxWaves; ++w)
-        before[w] = w < wave ? pass_counts[(size_t)w * nl + e] : 0;
+        before[w] = w < wave_s ? pass_counts[(size_t)w * nl + e] : 0;
       int32_t run = carry[parity * nl + e];
       const int32_t own = my_counts[e];
 #pragma unroll
