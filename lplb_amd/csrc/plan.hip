@@ -160,6 +160,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
   const int tid = threadIdx.x;
   constexpr int nt = WAVES * kWave;
   const int lane = tid % kWave, wave = tid / kWave;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, but known to be wave-uniform
   const int pid = blockIdx.x;
   const int n_workgroups = a.n_slices + 1;
   const int n_shares = a.sh.n_ranks * a.sh.D;
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     int32_t run = start[e];
 #pragma unroll
     for (int w = 0; w < WAVES; ++w)
-      run += w < wave ? counts[(size_t)w * nl + e] : 0;
+      run += w < wave_s ? counts[(size_t)w * nl + e] : 0;
     mine[e].next = run;
   }
   // The LP's shares decide how many tokens stay on the original.  Every thread that
