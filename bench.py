@@ -112,7 +112,8 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the plan; a run with --gpus > 1 is not supported "
-                 "(the path needs no collective: see DESIGN.md, sharding).")
+                 "(every rank plans its own tokens; the only exchange between ranks is the sum of the count "
+                 "vectors, which is not part of this measurement).")
 
     import torch
 
