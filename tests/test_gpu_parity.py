@@ -245,6 +245,59 @@ def test_solve_benchmark_configs(cuda, cfg, step_rule):
                    step_rule=step_rule)
 
 
+@pytest.mark.parametrize("topo", ["cube8", "ring8", "hyper16", "torus32"])
+def test_solve_adversarial_distributions(cuda, topo):
+    """Skewed, sparse, one-hot and nearly uniform count vectors, small and large totals.  On such inputs the
+    dense fp32 evaluation of the reference algorithm is itself up to 2e-4 (flows) / 1.3e-3 (objective) away
+    from its fp64 evaluation, so the yardstick here is the fp64 oracle: the GPU result (fp32 with an fp64
+    normal-equation solve) must be within the stated tolerances of it, and agree on feasibility."""
+    from lplb_amd import topology
+    from lplb_amd.mapping import build_redundancy_mapping
+    r2o, ep = {"cube8": (topology.CUBE_8P2E, 8), "ring8": (topology.RING_8P, 8),
+               "hyper16": (topology.HYPERCUBE_16P2E, 16), "torus32": (topology.torus_2d(8, 4), 32)}[topo]
+    r2o = np.asarray(r2o, np.int32)
+    nl = 256
+    shape = Shape(r2o, ep, nl, nl + r2o.shape[1] * ep)
+    solver = solver_for(shape)
+    rng = np.random.default_rng(99)
+
+    def draw(kind):
+        ranks = np.arange(1, nl + 1)
+        p = {"zipf1": 1.0 / ranks, "zipf2": 1.0 / ranks ** 2.0, "lognorm": rng.lognormal(0, 1.0, nl),
+             "near_uniform": 1 + rng.normal(0, 0.01, nl), "sparse": rng.random(nl) * (rng.random(nl) < 0.2) + 1e-6,
+             "one_hot": np.where(np.arange(nl) == rng.integers(nl), 1.0, 1e-3)}[kind]
+        p = rng.permutation(np.abs(p))
+        return rng.multinomial(int(rng.choice([1000, 65536, 1 << 22])), p / p.sum()).astype(np.int32)
+
+    flags_differ = checked = 0
+    worst = [0.0, 0.0]
+    for kind in ("zipf1", "zipf2", "lognorm", "near_uniform", "sparse", "one_hot"):
+        for _ in range(8):
+            hist = rng.integers(1, 1 << 20, size=nl)
+            phy2log, _, _ = build_redundancy_mapping(r2o, ep, nl, shape.n_physical, hist, n_nodes=1)
+            wl = draw(kind)
+            avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+            res, gw = solver.solve(dev(wl.reshape(shape.n_group, shape.G, shape.L), cuda), dev(r2o, cuda),
+                                   dev(phy2log, cuda), avail)
+            res = res.cpu().numpy()
+            o64, o_gw, o_avail = oracle.solve(wl, r2o, phy2log, shape.n_group, shape.C, shape.n_fixed, precision=64)
+            np.testing.assert_array_equal(gw.cpu().numpy().reshape(-1), o_gw)
+            if int(avail[0]) != o_avail:
+                flags_differ += 1
+                continue
+            if o_avail != shape.n_group:
+                assert np.all(res == 0.5)
+                continue
+            args = (r2o, phy2log, shape.n_group, shape.C)
+            flow = np.abs(oracle.edge_flows(wl, res, *args) - oracle.edge_flows(wl, o64, *args)).max() / float(wl.sum())
+            obj, obj64 = (oracle.rank_loads(wl, x, *args).max(axis=1) for x in (res, o64))
+            worst = [max(worst[0], flow), max(worst[1], float((np.abs(obj - obj64) / obj64).max()))]
+            checked += 1
+    print(f"{topo}: {checked} compared, worst flow {worst[0]:.1e} objective {worst[1]:.1e}, feasibility differs in {flags_differ}")
+    assert worst[0] <= FLOW_TOL and worst[1] <= OBJ_RTOL
+    assert flags_differ <= 2 and checked >= 40
+
+
 def test_solve_fallback_and_counter(cuda):
     """Infeasible / degenerate LPs give 0.5 everywhere and leave the counter alone;
     the counter accumulates across calls (minilp.cu:379-400)."""
