@@ -48,8 +48,10 @@ constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait 
 // [0] slices whose histogram row is published, [1] workgroups that have left,
 // [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
 // shares as 8-byte words (1 << 32) | float bits, 0 = not there yet.
-// From kTotalsAt on (own-histogram mode), the batch's tokens per logical expert, to
-// which every slice adds its row.
+// From kTotalsAt on (own-histogram mode), one 8-byte word per logical expert: the
+// batch's tokens of that expert in the high half and the number of slices that have
+// added theirs in the low half -- one atomic add per slice and expert delivers both,
+// so the reader needs no second round trip for a "done" counter.
 constexpr int kSharesAt = 16, kMaxShares = 256;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
 // One such block per stream that has run a plan (the compute stream, a warm-up
@@ -57,7 +59,7 @@ constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
 // do not share counters.  A launch takes at most a quarter of the CUs: up to three
 // plans that really execute at the same time are all resident; with four or more,
 // workgroups could wait for workgroups that cannot start.
-constexpr int kSlotInts = kTotalsAt + kMaxTotals, kSyncSlots = 8;
+constexpr int kSlotInts = kTotalsAt + 2 * kMaxTotals, kSyncSlots = 8;
 static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
 static bool g_cooperative = true;
 
@@ -130,7 +132,7 @@ __device__ inline void leave(int *sync, int n_workgroups, int n_shares, int n_to
   unsigned long long *shares = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
   for (int i = threadIdx.x; i < n_shares; i += blockDim.x)
     __hip_atomic_store(shares + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  for (int i = threadIdx.x; i < n_totals; i += blockDim.x)
+  for (int i = threadIdx.x; i < 2 * n_totals; i += blockDim.x)
     agent_store(sync + kTotalsAt + i, 0);
   if (threadIdx.x == 0) {
     agent_store(sync + 0, 0);
@@ -181,22 +183,35 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
       __syncthreads();
       sa.counts_ready = &counts_ready;
       if (wave == sa.n_units) {
-        if (lane == 0)
-          wait_for(a.sync, 0, a.n_slices);
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        for (int e0 = lane; e0 < nl; e0 += 8 * kWave) {
-          int32_t t[8];
+        // Poll the totals until every expert's word says that all slices have added
+        // theirs (plain loads after an acquire fence: they can be batched).
+        const unsigned long long *words = reinterpret_cast<const unsigned long long *>(a.sync + kTotalsAt);
+        for (int polls = 0;; ++polls) {
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+          bool all_in = true;
+          for (int e0 = lane; e0 < nl; e0 += 8 * kWave) {
+            unsigned long long t[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k)
-            t[k] = a.sync[kTotalsAt + min(e0 + k * kWave, nl - 1)];
+            for (int k = 0; k < 8; ++k)
+              t[k] = words[min(e0 + k * kWave, nl - 1)];
 #pragma unroll
-          for (int k = 0; k < 8; ++k)
-            if (e0 + k * kWave < nl) {
-              staged[e0 + k * kWave] = (float)t[k];
-              a.totals[e0 + k * kWave] = t[k];
+            for (int k = 0; k < 8; ++k) {
+              all_in = all_in && (uint32_t)t[k] == (uint32_t)a.n_slices;
+              if (e0 + k * kWave < nl)
+                staged[e0 + k * kWave] = (float)(uint32_t)(t[k] >> 32);
             }
+          }
+          if (__all(all_in))
+            break;
+          if (polls >= kMaxPolls) {
+            if (lane == 0)
+              __hip_atomic_fetch_add(a.sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
         }
+        for (int e = lane; e < nl; e += kWave)   // this GPU's totals, for the caller
+          a.totals[e] = (int32_t)staged[e];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
           __hip_atomic_store(&counts_ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -253,8 +268,10 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     for (int w = 0; w < WAVES; ++w)
       h += counts[(size_t)w * nl + e];
     agent_store(a.rows + (int64_t)pid * nl + e, h);
-    if (a.local_counts && h != 0)
-      __hip_atomic_fetch_add(a.sync + kTotalsAt + e, h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (a.local_counts)
+      __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + e,
+                             ((unsigned long long)(uint32_t)h << 32) | 1ull, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
   }
   __builtin_amdgcn_s_waitcnt(0);   // the row has left this CU
   __syncthreads();
