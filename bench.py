@@ -47,6 +47,8 @@ def event_times_us(fn, n, warmup, torch):
     for _ in range(warmup):
         fn()
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+    for e in ev:
+        e.record()
     torch.cuda.synchronize()
     ev[0].record()
     for i in range(n):
@@ -186,6 +188,8 @@ def main() -> None:
     for _ in range(args.warmup):
         plan()
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    for e in ev:          # torch creates the HIP event at the first record: keep that out of the timed region
+        e.record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ev[0].record()
