@@ -41,6 +41,22 @@ LaunchEvents take_launch_events();
 // Compute units of the current device (looked up once per device); 0 if the query fails.
 int current_device_cu_count();
 
+// Lets `kernel` use up to `bytes` of dynamic LDS (above the 64 KiB default the
+// runtime has to be told, once per kernel and device).
+template <typename Kernel> hipError_t allow_dynamic_lds(Kernel kernel, int bytes) {
+  static bool told[64];
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess)
+    return err;
+  if (dev < 0 || dev >= 64 || !told[dev]) {
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err == hipSuccess && dev >= 0 && dev < 64)
+      told[dev] = true;
+  }
+  return err;
+}
+
 // Every kernel of the library is launched through here.  If the calling thread
 // armed a pair of events, the launch records the kernel's own begin and end
 // timestamps into them (not the time the launch was enqueued).

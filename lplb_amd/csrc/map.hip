@@ -190,11 +190,9 @@ static size_t map_lds_bytes(int n_logical, int w) {
 template <int K, bool WRAP>
 static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
   if (lds > 64 * 1024) {
-    // above the default limit the kernel has to be told once per process
-    static hipError_t raised = hipFuncSetAttribute(reinterpret_cast<const void *>(&redirect_indices<K, WRAP>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (raised != hipSuccess)
-      return raised;
+    const hipError_t err = allow_dynamic_lds(&redirect_indices<K, WRAP>, 160 * 1024);
+    if (err != hipSuccess)
+      return err;
   }
   launch(redirect_indices<K, WRAP>, grid, block, lds, s, a);
   return hipGetLastError();

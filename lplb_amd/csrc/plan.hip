@@ -352,11 +352,9 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
 template <int GM, int DM, bool EXACT, int K, int WAVES>
 static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t s) {
   if (lds > 64 * 1024) {
-    static hipError_t raised =
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&plan_in_one_launch<GM, DM, EXACT, K, WAVES>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kPlanLdsLimit);
-    if (raised != hipSuccess)
-      return raised;
+    const hipError_t err = allow_dynamic_lds(&plan_in_one_launch<GM, DM, EXACT, K, WAVES>, kPlanLdsLimit);
+    if (err != hipSuccess)
+      return err;
   }
   launch(plan_in_one_launch<GM, DM, EXACT, K, WAVES>, dim3(a.n_slices + 1), dim3(WAVES * kWave), lds, s, a);
   return hipGetLastError();
