@@ -4,62 +4,48 @@
 
 namespace lplb {
 
-// WAVES: waves per workgroup; a bigger workgroup only means fewer of them to
-// dispatch and fewer increments of the feasibility counter.
-template <int GM, int DM, bool EXACT, int ROWS, int WAVES>
-__global__ __launch_bounds__(kWave * WAVES) void solve_groups(SolveArgs a) {
-  extern __shared__ float staged_all[];   // a.staged_stride floats per LP of this workgroup
-  __shared__ int rep_of_edge_all[kWave * WAVES];
-  __shared__ int feasible_in_workgroup;
-  if (WAVES > 1) {
-    if (threadIdx.x == 0)
-      feasible_in_workgroup = 0;
-    __syncthreads();
-  }
-  const int wave = threadIdx.x / kWave;
-  const int n_ok = solve_lp<GM, DM, EXACT, ROWS>(a, (blockIdx.x * WAVES + wave) * ROWS,
-                                                 staged_all + (size_t)wave * ROWS * a.staged_stride,
-                                                 rep_of_edge_all + wave * kWave);
-  // Increments of the one counter queue up behind each other in memory (about
-  // 10 ns each), so the waves of a workgroup add up in LDS first.
-  if (WAVES == 1) {
-    if (threadIdx.x == 0 && n_ok > 0)
-      atomicAdd(a.avail, n_ok);
-  } else {
-    if (threadIdx.x % kWave == 0 && n_ok > 0)
-      atomicAdd(&feasible_in_workgroup, n_ok);
-    __syncthreads();   // every wave gets here: none leaves early
-    if (threadIdx.x == 0 && feasible_in_workgroup > 0)
-      atomicAdd(a.avail, feasible_in_workgroup);
-  }
+// One wave per workgroup; ROWS LPs per wave.
+//
+// Feasibility counter: updates of one address queue up behind each other in memory
+// (about 10 ns each: 2048 waves that each add their result take 20 us longer than
+// the arithmetic).  So the first thread of the grid counts every LP of the launch as
+// feasible with one add, and a wave takes back the LPs of its own that failed -- rare,
+// and the sum is the same.
+template <int GM, int DM, bool EXACT, int ROWS>
+__global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
+  extern __shared__ float staged_all[];   // a.staged_stride floats per LP of this wave
+  __shared__ int rep_of_edge[kWave];
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    atomicAdd(a.avail, a.n_units);
+  const int first_unit = blockIdx.x * ROWS;
+  const int n_ok = solve_lp<GM, DM, EXACT, ROWS>(a, first_unit, staged_all, rep_of_edge);
+  const int n_mine = min(max(a.n_units - first_unit, 0), ROWS);
+  if (threadIdx.x == 0 && n_ok < n_mine)
+    atomicAdd(a.avail, n_ok - n_mine);
 }
 
-// How many LPs share a wave and how many waves a workgroup, by batch size:
-//  * up to kLoneWaves LPs: one wave each, alone in its workgroup (lowest latency;
-//    every wave pays its own increment of the feasibility counter);
-//  * more: workgroups of kWaves waves that combine their increments;
-//  * from kPackFrom LPs on, shapes with G <= 16 and G * D <= 16 put four LPs into
-//    each wave, which takes 2 us longer per wave and a quarter of the waves.
-constexpr int kLoneWaves = 64, kWaves = 4, kPackFrom = 1024;
+// One LP per wave has the lowest latency (8 us at (8, 2)) and is the fastest form
+// until the waves outnumber the SIMDs; from kPackFrom LPs on, shapes with G <= 16 and
+// G * D <= 16 put four LPs into each wave (10.4 us per wave, a quarter of the waves).
+// Measured at (8, 2): 1024 LPs 8.8 us unpacked; 2048 LPs 12.9 us unpacked, 11.4 us
+// packed; 16384 LPs 73 us unpacked, 31 us packed.
+constexpr int kPackFrom = 1536;
 constexpr int kLdsLimit = 64 * 1024 - 2048;
 
-template <int GM, int DM, bool EXACT, int ROWS, int WAVES>
+template <int GM, int DM, bool EXACT, int ROWS>
 static void launch_variant(SolveArgs a, hipStream_t s) {
-  const int per_wg = ROWS * WAVES;
-  const size_t lds = (size_t)per_wg * a.n_experts * sizeof(float);
+  const size_t lds = (size_t)ROWS * a.n_experts * sizeof(float);
   a.staged_stride = lds <= kLdsLimit ? a.n_experts : 0;
-  launch(solve_groups<GM, DM, EXACT, ROWS, WAVES>, dim3((a.n_units + per_wg - 1) / per_wg),
-         dim3(kWave * WAVES), a.staged_stride ? lds : 0, s, a);
+  launch(solve_groups<GM, DM, EXACT, ROWS>, dim3((a.n_units + ROWS - 1) / ROWS), dim3(kWave),
+         a.staged_stride ? lds : 0, s, a);
 }
 
 template <int GM, int DM, bool EXACT> static void launch_exactness(const SolveArgs &a, hipStream_t s) {
   if constexpr (GM <= kRowLanes && GM * DM <= kRowLanes) {
     if (a.n_units >= kPackFrom)
-      return launch_variant<GM, DM, EXACT, 4, kWaves>(a, s);
+      return launch_variant<GM, DM, EXACT, 4>(a, s);
   }
-  if (a.n_units > kLoneWaves)
-    return launch_variant<GM, DM, EXACT, 1, kWaves>(a, s);
-  launch_variant<GM, DM, EXACT, 1, 1>(a, s);
+  launch_variant<GM, DM, EXACT, 1>(a, s);
 }
 
 template <int GM, int DM> static void launch_solver(const SolveArgs &a, hipStream_t s) {

@@ -342,15 +342,15 @@ def _shifted_ring(g, shifts):
 
 
 @pytest.mark.parametrize("name,r2o,ep,n_logical,n_inst", [
-    ("cube8x2", None, 8, 256, 1029),                         # exact instantiation, last wave part full
-    ("ring8x1", _shifted_ring(8, [1]), 8, 128, 1026),
-    ("ring6x2_padded", _shifted_ring(6, [1, 2]), 6, 60, 1025),  # rounded up to the 8 x 2 instantiation
-    ("ring16x1", _shifted_ring(16, [1]), 32, 256, 515),      # two groups per instance
+    ("cube8x2", None, 8, 256, 1541),                         # exact instantiation, last wave part full
+    ("ring8x1", _shifted_ring(8, [1]), 8, 128, 1538),
+    ("ring6x2_padded", _shifted_ring(6, [1, 2]), 6, 60, 1537),  # rounded up to the 8 x 2 instantiation
+    ("ring16x1", _shifted_ring(16, [1]), 32, 256, 771),      # two groups per instance
 ])
 def test_solve_batched_four_per_wave(cuda, name, r2o, ep, n_logical, n_inst):
-    """From 1024 LPs on, small shapes are solved four to a wave (one per 16-lane row), and
-    above 64 LPs the waves share workgroups.  Those kernels must agree with the lone-wave
-    kernel (batches up to 64) and with the oracle, also in a wave that is only partly filled."""
+    """From 1536 LPs on, small shapes are solved four to a wave (one per 16-lane row).  That kernel
+    must agree with the one-LP-per-wave kernel (smaller batches) and with the oracle, also in a
+    wave that is only partly filled, and the feasibility counter must add up either way."""
     from lplb_amd import topology
     from lplb_amd.mapping import build_redundancy_mapping
     r2o = topology.CUBE_8P2E if r2o is None else r2o
@@ -366,14 +366,9 @@ def test_solve_batched_four_per_wave(cuda, name, r2o, ep, n_logical, n_inst):
     packed, gws = solver.solve_batched(wl, d_r2o, d_p2l, avail, want_global=True)
     n_ok = int(avail[0])
     avail.zero_()
-    chunk = 64 // shape.n_group
+    chunk = 500 // shape.n_group
     by_wave = torch.cat([solver.solve_batched(wl[i:i + chunk], d_r2o, d_p2l, avail) for i in range(0, n_inst, chunk)])
     assert int(avail[0]) == n_ok
-    avail.zero_()
-    chunk = 600 // shape.n_group
-    shared = torch.cat([solver.solve_batched(wl[i:i + chunk], d_r2o, d_p2l, avail) for i in range(0, n_inst, chunk)])
-    assert int(avail[0]) == n_ok
-    assert torch.equal(shared, by_wave)      # same arithmetic, only the workgroup size differs
     assert packed.shape == by_wave.shape == (n_inst, shape.n_group, shape.G, shape.D)
     # b_i is summed by a different number of lanes in the two kernels, so the shares differ by
     # rounding, amplified where the LP is ill-conditioned (a long ring): compare the flows.
