@@ -718,6 +718,31 @@ def test_plans_on_two_streams(cuda, cooperative):
         _native.set_plan_cooperative(True)
 
 
+def test_one_launch_plan_while_another_stream_fills_the_gpu(cuda):
+    """The workgroups of the one-launch plan wait for each other; they must still all get their turn when
+    another stream keeps every CU busy (here with matrix products), and no wait may run out."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])
+    want = want.clone()
+    torch.cuda.synchronize()
+    a = torch.randn(4096, 4096, device=cuda, dtype=torch.bfloat16)
+    b = torch.randn(4096, 4096, device=cuda, dtype=torch.bfloat16)
+    busy, planning = torch.cuda.Stream(), torch.cuda.Stream()
+    for rep in range(10):
+        with torch.cuda.stream(busy):
+            for _ in range(4):
+                c = a @ b
+        with torch.cuda.stream(planning):
+            outs = [solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])[0]
+                    for _ in range(4)]
+        torch.cuda.synchronize()
+        assert all(torch.equal(o, want) for o in outs), rep
+        del c
+    assert _native.plan_sync_timeouts() == 0
+
+
 def test_kernel_timestamp_hook(cuda):
     import ctypes
     inp, shape, solver, t = _plan_setup(cuda, "cpu_ref_ep8")
