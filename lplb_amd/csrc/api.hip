@@ -1,4 +1,5 @@
 // Error reporting and version query of the C ABI.
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -33,17 +34,17 @@ long long *g_phase_clocks = nullptr;
 static thread_local LaunchEvents g_launch_events;
 
 int current_device_cu_count() {
-  static int cus_of[64];
+  static std::atomic<int> cus_of[64];
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
     return 0;
-  if (cus_of[dev] == 0) {
-    int n = 0;
+  int n = cus_of[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
       return 0;
-    cus_of[dev] = n;
+    cus_of[dev].store(n, std::memory_order_relaxed);
   }
-  return cus_of[dev];
+  return n;
 }
 
 LaunchEvents take_launch_events() {

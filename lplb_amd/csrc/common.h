@@ -5,6 +5,8 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/lplb_hip.h"
 
 namespace lplb {
@@ -44,15 +46,15 @@ int current_device_cu_count();
 // Lets `kernel` use up to `bytes` of dynamic LDS (above the 64 KiB default the
 // runtime has to be told, once per kernel and device).
 template <typename Kernel> hipError_t allow_dynamic_lds(Kernel kernel, int bytes) {
-  static bool told[64];
+  static std::atomic<bool> told[64];
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess)
     return err;
-  if (dev < 0 || dev >= 64 || !told[dev]) {
+  if (dev < 0 || dev >= 64 || !told[dev].load(std::memory_order_acquire)) {
     err = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (err == hipSuccess && dev >= 0 && dev < 64)
-      told[dev] = true;
+      told[dev].store(true, std::memory_order_release);
   }
   return err;
 }

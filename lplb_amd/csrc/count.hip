@@ -34,9 +34,13 @@ __global__ __launch_bounds__(1024) void slice_histogram(
 
   const int64_t begin = slice_begin(n, per, p);
   const int64_t end = slice_begin(n, per, p + 1);
-  // Slices start on multiples of 256 indices, so pairs are 16-byte aligned.
-  const int64_t n_pairs = (end - begin) >> 1;
-  const longlong2 *pairs = reinterpret_cast<const longlong2 *>(idx + begin);
+  // Pairs are loaded 16 bytes at a time.  Slices start on multiples of 256 indices,
+  // so a slice starts on a 16-byte boundary unless the array itself sits at an odd
+  // multiple of 8 bytes (a view that starts inside a tensor); then its first index
+  // is counted alone.
+  const int64_t head = (begin < end && (reinterpret_cast<uintptr_t>(idx + begin) & 8)) ? 1 : 0;
+  const int64_t n_pairs = (end - begin - head) >> 1;
+  const longlong2 *pairs = reinterpret_cast<const longlong2 *>(idx + begin + head);
   for (int64_t i0 = tid; i0 < n_pairs; i0 += (int64_t)nt * kLoadsInFlight) {
     longlong2 v[kLoadsInFlight];
 #pragma unroll
@@ -50,7 +54,9 @@ __global__ __launch_bounds__(1024) void slice_histogram(
       count_one(hist, v[u].y, n_experts);
     }
   }
-  if (tid == 0 && ((end - begin) & 1))
+  if (tid == 0 && head)
+    count_one(hist, idx[begin], n_experts);
+  if (tid == 0 && ((end - begin - head) & 1))
     count_one(hist, idx[end - 1], n_experts);
   __syncthreads();
   int32_t *row = counts + (int64_t)p * n_experts;
@@ -140,8 +146,8 @@ extern "C" int lplb_count_idx(const int64_t *idx, int64_t n_elements,
                "count_idx: n_experts=%d n_blocks=%d must be positive", n_experts, n_blocks);
   LPLB_REQUIRE(counts_by_block != nullptr && (idx != nullptr || n_elements == 0), LPLB_EINVAL,
                "count_idx: null pointer");
-  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL,
-               "count_idx: idx must be 16-byte aligned");
+  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 7) == 0, LPLB_EINVAL,
+               "count_idx: idx must be 8-byte aligned");
   return enqueue_count(idx, n_elements, n_experts, n_blocks, counts_by_block,
                        static_cast<hipStream_t>(stream), /*any_order=*/false);
 }

@@ -36,6 +36,7 @@
 // these limits switch this path off with lplb_plan_set_cooperative(0).
 #include "map_kernel.h"
 #include "solve_kernel.h"
+#include <atomic>
 #include <mutex>
 
 namespace lplb {
@@ -61,7 +62,7 @@ constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
 // workgroups could wait for workgroups that cannot start.
 constexpr int kSlotInts = kTotalsAt + 2 * kMaxTotals, kSyncSlots = 8;
 static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
-static bool g_cooperative = true;
+static std::atomic<bool> g_cooperative{true};   // any thread may flip it while others plan
 
 struct PlanArgs {
   const int64_t *idx;
@@ -407,21 +408,21 @@ static int sync_slot_of(hipStream_t s) {
   return used++;
 }
 
-// Per-device address of the counters and CU count, looked up once.
+// Per-device address of the counters and CU count, looked up once (threads that race
+// for the first look-up store the same values).
 static int plan_device_state(int **sync, int *n_cus) {
-  static int *sync_of[64];
-  static int cus_of[64];
+  static std::atomic<int *> sync_of[64];
   int dev = -1;
   LPLB_HIP_TRY(hipGetDevice(&dev));
   LPLB_REQUIRE(dev >= 0 && dev < 64, LPLB_EUNSUPPORTED, "plan: device ordinal %d", dev);
-  if (!sync_of[dev]) {
-    int *p = nullptr;
+  int *p = sync_of[dev].load(std::memory_order_acquire);
+  if (!p) {
     LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_plan_sync)));
-    LPLB_HIP_TRY(hipDeviceGetAttribute(&cus_of[dev], hipDeviceAttributeMultiprocessorCount, dev));
-    sync_of[dev] = p;
+    sync_of[dev].store(p, std::memory_order_release);
   }
-  *sync = sync_of[dev];
-  *n_cus = cus_of[dev];
+  *sync = p;
+  *n_cus = current_device_cu_count();
+  LPLB_REQUIRE(*n_cus > 0, LPLB_EHIP, "plan: cannot read the CU count of device %d", dev);
   return LPLB_OK;
 }
 
@@ -536,7 +537,7 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
   LPLB_REQUIRE(counts_by_block != nullptr, LPLB_EINVAL, "plan: null counts_by_block");
   LPLB_REQUIRE(n_elements >= 0 && n_elements <= INT32_MAX && (idx || n_elements == 0), LPLB_EINVAL,
                "plan: bad idx / n_elements=%lld", (long long)n_elements);
-  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 15) == 0, LPLB_EINVAL, "plan: idx must be 16-byte aligned");
+  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 7) == 0, LPLB_EINVAL, "plan: idx must be 8-byte aligned");
   LPLB_REQUIRE(r2o && o2r && phy2log && o_weight && avail_num && (out || n_elements == 0), LPLB_EINVAL,
                "plan: null pointer");
   LPLB_REQUIRE(step_rule == LPLB_STEP_REFERENCE_WINDOW || step_rule == LPLB_STEP_FULL_MAX, LPLB_EINVAL,

@@ -411,7 +411,10 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // The only serial chain is pivot -> reciprocal -> f -> entry (c+1, c+1) -> next
     // pivot; it is written out in that order, with the rest of column step c (which
     // nothing waits for) placed between the links of the next reciprocal, because
-    // the compiler keeps the order it is given here.
+    // the compiler keeps the order it is given here.  (Broadcasting the far columns
+    // of row c through LDS instead of v_readlane halves their instruction count at
+    // 32 ranks, but puts an LDS write -> read round trip into every step of the chain:
+    // measured 45 us against 34 us.)
     double my_pivot = 1.0;
     double pivot = lp_bcast<ROWS, 0>(S[0]);
     double rinv = rcp_f64(pivot);

@@ -411,6 +411,34 @@ def test_run_matches_oracle_chain(cuda, cfg, mask):
     np.testing.assert_array_equal(out.cpu().numpy(), want)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("offset", [1, 3, 256, 257])
+def test_run_on_a_view_that_starts_inside_a_tensor(cuda, offset):
+    """A contiguous view whose first element sits at an odd multiple of 8 bytes is a legal
+    input of the reference (csrc/plugin.cpp:582-584 asks for int64 and contiguity only)."""
+    c = synth.CONFIGS["cpu_ref_ep8"]
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    rng = np.random.default_rng(900 + offset)
+    whole = rng.integers(-1, c.n_logical, size=offset + 5001, dtype=np.int64)
+    d_whole = dev(whole, cuda)
+    d_idx = d_whole[offset:]
+    assert d_idx.is_contiguous() and d_idx.data_ptr() == d_whole.data_ptr() + 8 * offset
+    idx = whole[offset:]
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    phy2log = planner.phy2log.cpu().numpy()
+    for n_sms in (2, 16, 64):
+        by_sm = oracle.count_idx(idx, c.n_logical, n_sms)
+        local, by_sm_gpu = planner.count_workload(d_idx, n_sms)
+        np.testing.assert_array_equal(by_sm_gpu.cpu().numpy(), by_sm)
+        np.testing.assert_array_equal(local.cpu().numpy().ravel(), by_sm[-1])
+        avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+        out = planner.run(d_idx, avail, n_sms)
+        o_weight, _ = planner.solve_probs(local, torch.zeros(1, dtype=torch.int32, device=cuda))
+        want = oracle.map_idx(idx, o_weight.cpu().numpy(), by_sm, shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+        np.testing.assert_array_equal(out.cpu().numpy(), want)
+    np.testing.assert_array_equal(d_whole.cpu().numpy(), whole)   # nothing outside the view was touched
+
+
 @pytest.mark.parametrize("kind", ["empty", "all_masked", "one_token", "odd_length", "one_expert_only"])
 def test_run_edge_inputs(cuda, kind):
     """Degenerate batches go through the same three kernels (tests/test_idx_processing.py of the
