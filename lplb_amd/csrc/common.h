@@ -6,6 +6,8 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 #include "../../include/lplb_hip.h"
 
@@ -105,6 +107,15 @@ __host__ __device__ inline int64_t slice_len(int64_t n, int parts) {
 __host__ __device__ inline int64_t slice_begin(int64_t n, int64_t per, int p) {
   int64_t v = per * p;
   return v < n ? v : n;
+}
+
+// Calls f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>):
+// a loop whose index is a constant expression.
+template <typename F, int... I> __device__ inline void static_for_impl(F &f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ inline void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // ---- wave64 primitives -----------------------------------------------------

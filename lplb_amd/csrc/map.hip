@@ -146,22 +146,29 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
     // every wave clears its row of the other half for the next pass.
     const int32_t *pass_counts = counts + (size_t)parity * n_waves * nl;
     int32_t *other_counts = counts + ((size_t)(parity ^ 1) * n_waves + wave) * nl;
-    for (int e = lane; e < nl; e += kWave) {
-      // all reads in flight before the first add
-      int32_t before[kMaxWaves];
+    // The code is specialised by the number of earlier waves (wave-uniform), so that
+    // the inner loop is straight-line: exactly that many reads, no branches.
+    static_for<kMaxWaves>([&](auto wc) {
+      constexpr int kEarlier = decltype(wc)::value;
+      if (wave_s != kEarlier)
+        return;
+      for (int e = lane; e < nl; e += kWave) {
+        // all reads in flight before the first add
+        int32_t before[kEarlier + 1];
 #pragma unroll
-      for (int w = 0; w < kMaxWaves; ++w)
-        before[w] = w < wave_s ? pass_counts[(size_t)w * nl + e] : 0;
-      int32_t run = carry[parity * nl + e];
-      const int32_t own = my_counts[e];
+        for (int w = 0; w < kEarlier; ++w)
+          before[w] = pass_counts[(size_t)w * nl + e];
+        int32_t run = carry[parity * nl + e];
+        const int32_t own = my_counts[e];
 #pragma unroll
-      for (int w = 0; w < kMaxWaves; ++w)
-        run += before[w];
-      mine[e].next = run;
-      if (wave == n_waves - 1)
-        carry[(parity ^ 1) * nl + e] = run + own;
-      other_counts[e] = 0;
-    }
+        for (int w = 0; w < kEarlier; ++w)
+          run += before[w];
+        mine[e].next = run;
+        if (kEarlier == n_waves - 1)
+          carry[(parity ^ 1) * nl + e] = run + own;
+        other_counts[e] = 0;
+      }
+    });
     __builtin_amdgcn_wave_barrier();
     LPLB_MAP_STAMP(4);
     // Phase C.

@@ -31,8 +31,6 @@
 // factorisation shows on nearly balanced loads.  Everything else is fp32.
 #pragma once
 #include "common.h"
-#include <type_traits>
-#include <utility>
 
 namespace lplb {
 
@@ -100,15 +98,6 @@ template <int W> __device__ inline float reduce_max(float v) {
 __device__ inline double rcp_f64(double a) {
   double r = __builtin_amdgcn_rcp(a);
   return __builtin_fma(__builtin_fma(-a, r, 1.0), r, r);
-}
-
-// Calls f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>):
-// a loop whose index is a constant expression, as the DPP controls need.
-template <typename F, int... I> __device__ inline void static_for_impl(F &f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F> __device__ inline void static_for(F &&f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // ---- one LP per wave (ROWS == 1) or one LP per 16-lane DPP row (ROWS == 4) ----
