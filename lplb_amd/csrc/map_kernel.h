@@ -57,15 +57,24 @@ __device__ inline void set_original(ExpertEntry *table, const RedirectShape &sh,
   if (le >= 0 && le < sh.n_logical)
     table[le].original = (e / sh.L) * sh.P + (e % sh.L);
 }
-// Replica slot `local` of EP rank ep_rank copies logical expert le, whose original
-// keeps `share` of its tokens; the copy lives on group rank `host`.
+// Replica slot `local` of EP rank ep_rank copies logical expert le; the copy lives on
+// group rank `host`.
+__device__ inline void set_replica_slot(int32_t *replica, const RedirectShape &sh, int ep_rank, int local, int le,
+                                        int host) {
+  if (le >= 0 && le < sh.n_logical)
+    replica[le] = ((ep_rank / sh.G) * sh.G + host + 1) * sh.P - sh.C * sh.D + local;
+}
+// Tokens of an expert with `total` tokens that stay on its original when the original
+// keeps `share` of them: the fp32 product truncated toward zero (saturating, NaN -> 0).
+__device__ inline int32_t expected_on_original(float share, int32_t total) {
+  return __float2int_rz(share * (float)total);
+}
+// Both at once.
 __device__ inline void set_replica(ExpertEntry *table, int32_t *replica, const RedirectShape &sh, int ep_rank,
                                    int local, int le, float share, int host) {
-  if (le >= 0 && le < sh.n_logical) {
-    // fp32 product truncated toward zero (saturating, NaN -> 0)
-    table[le].expected = __float2int_rz(share * (float)table[le].total);
-    replica[le] = ((ep_rank / sh.G) * sh.G + host + 1) * sh.P - sh.C * sh.D + local;
-  }
+  if (le >= 0 && le < sh.n_logical)
+    table[le].expected = expected_on_original(share, table[le].total);
+  set_replica_slot(replica, sh, ep_rank, local, le, host);
 }
 
 // How many of an expert's `total` tokens stay on the original:
@@ -106,15 +115,17 @@ __device__ inline void emit_physical_counts(const ExpertEntry *table, const int3
 // One token of a 64-index chunk: lanes holding the same expert find each other
 // through the wave's 64-bit bitmap for that expert; the rank among those peers is a
 // popcount of lower lanes and the last peer advances the wave's ordinal.  Returns
-// the physical expert (-1 for e < 0).  All lanes of the wave call it together and
-// put a wave barrier between chunks.
+// the token's hash (499 k + 41) mod total (minilp.cu:505) and, in x, its expert's
+// entry; neither is defined for e < 0.  All lanes of the wave call it together and
+// put a wave barrier between chunks.  It does not read x.expected, so it may run
+// before the LP's shares are known.
 template <bool WRAP>
-__device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntry *table, const int32_t *replica,
-                                         unsigned long long my_bit) {
+__device__ inline int32_t hash_of_token(int e, WaveSlot *mine, const ExpertEntry *table, unsigned long long my_bit,
+                                        ExpertEntry &x) {
   const bool valid = e >= 0;
   if (valid)
     atomicOr(&mine[e].bits, my_bit);
-  int64_t o = -1;
+  int32_t h = 0;
   if (valid) {
     const i32x4 sraw = *reinterpret_cast<const i32x4 *>(&mine[e]);
     const i32x4 xraw = *reinterpret_cast<const i32x4 *>(&table[e]);
@@ -122,14 +133,23 @@ __device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntr
     const int rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
     const int cnt = __popc(peers_lo) + __popc(peers_hi);
     const int32_t k = sraw.x + rank;
-    ExpertEntry x;
     x.total = xraw.x; x.magic = (uint32_t)xraw.y; x.expected = xraw.z; x.original = xraw.w;
-    // (k * 499 + 41) % total in int32 arithmetic (minilp.cu:505)
-    const int32_t h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
-    o = h >= x.expected ? replica[e] : x.original;
+    h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
     if (rank == cnt - 1)   // last peer: advance the ordinal, clear the bitmap
       *reinterpret_cast<i32x4 *>(&mine[e]) = i32x4{k + 1, 0, 0, 0};
   }
+  return h;
+}
+
+// The physical expert of a token of expert e with hash h (-1 for e < 0).
+template <bool WRAP>
+__device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntry *table, const int32_t *replica,
+                                         unsigned long long my_bit) {
+  ExpertEntry x;
+  const int32_t h = hash_of_token<WRAP>(e, mine, table, my_bit, x);
+  int64_t o = -1;
+  if (e >= 0)
+    o = h >= x.expected ? replica[e] : x.original;
   return o;
 }
 

@@ -244,6 +244,14 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
   const int64_t end = slice_begin(a.n, a.per, pid + 1);
 
   LPLB_PLAN_STAMP(0);
+  // Small table reads that depend on nothing go out first; they are used much later.
+  const int cd = a.sh.C * a.sh.D, n_sets = a.sh.n_ranks * cd;
+  const int le_of_tid = tid < nl ? a.phy2log[(tid / a.sh.L) * a.sh.P + (tid % a.sh.L)] : -1;
+  // first (usually only) replicated expert set of this thread
+  const bool set0 = tid < n_sets;
+  const int rank0 = set0 ? tid / cd : 0, local0 = set0 ? tid % cd : 0;
+  const int rle0 = set0 ? a.phy2log[rank0 * a.sh.P + local0] : -1;
+  const int host0 = set0 ? a.o2r[(rank0 % a.sh.G) * a.sh.D + local0 % a.sh.D] : 0;
   int32_t ev[K];   // expert ids, -1 for masked / out-of-range / past the end
 #pragma unroll
   for (int c = 0; c < K; ++c) {
@@ -307,24 +315,60 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
       a.totals[e] = t;
   }
   __syncthreads();
-  for (int e = tid; e < nl; e += nt)
+  if (tid < nl)
+    set_original(table, a.sh, tid, le_of_tid);
+  for (int e = tid + nt; e < nl; e += nt)
     set_original(table, a.sh, e, a.phy2log[(e / a.sh.L) * a.sh.P + (e % a.sh.L)]);
   LPLB_PLAN_STAMP(7);
-  // each wave's starting ordinals: tokens before this slice + those of the waves before it
-  for (int e = lane; e < nl; e += kWave) {
-    int32_t run = start[e];
+  // each wave's starting ordinals: tokens before this slice + those of the waves before
+  // it; specialised by the (wave-uniform) number of those, so that the loop is
+  // straight-line with exactly that many reads
+  static_for<WAVES>([&](auto wc) {
+    constexpr int kEarlier = decltype(wc)::value;
+    if (wave_s != kEarlier)
+      return;
+    for (int e = lane; e < nl; e += kWave) {
+      int32_t before[kEarlier + 1];
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
-      run += w < wave_s ? counts[(size_t)w * nl + e] : 0;
-    mine[e].next = run;
-  }
-  // The LP's shares decide how many tokens stay on the original.  Every thread that
-  // needs one polls it itself: value and "valid" arrive in the same 8-byte word.
+      for (int w = 0; w < kEarlier; ++w)
+        before[w] = counts[(size_t)w * nl + e];
+      int32_t run = start[e];
+#pragma unroll
+      for (int w = 0; w < kEarlier; ++w)
+        run += before[w];
+      mine[e].next = run;
+    }
+  });
+  // The LP's shares decide how many tokens stay on the original, and nothing else:
+  // replica slots, ordinals and hashes are worked out while the LP is still running,
+  // so that one multiplication and one comparison per token are left for afterwards.
   LPLB_PLAN_STAMP(3);
-  const int cd = a.sh.C * a.sh.D;
   const unsigned long long *shares = reinterpret_cast<const unsigned long long *>(a.sync + kSharesAt);
-  for (int i = tid; i < a.sh.n_ranks * cd; i += nt) {
-    const int ep_rank = i / cd, local = i % cd, d = local % a.sh.D;
+  int le0 = -1;
+  int32_t total0 = 0;
+  if (set0) {
+    set_replica_slot(replica, a.sh, rank0, local0, rle0, host0);
+    if (rle0 >= 0 && rle0 < nl) {
+      le0 = rle0;
+      total0 = table[le0].total;
+    }
+  }
+  for (int i = tid + nt; i < n_sets; i += nt) {
+    const int ep_rank = i / cd, local = i % cd;
+    set_replica_slot(replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local],
+                     a.o2r[(ep_rank % a.sh.G) * a.sh.D + local % a.sh.D]);
+  }
+  __builtin_amdgcn_wave_barrier();   // the wave's starting ordinals above are read by other lanes below
+  int32_t h[K];
+#pragma unroll
+  for (int c = 0; c < K; ++c) {
+    ExpertEntry unused;
+    h[c] = hash_of_token<false>(ev[c], mine, table, my_bit, unused);
+    __builtin_amdgcn_wave_barrier();
+  }
+  // Every thread that needs a share polls it itself: value and "valid" arrive in the
+  // same 8-byte word.
+  auto share_of = [&](int ep_rank, int d) {
     unsigned long long word = 0;
     int polls = 0;
     while ((word = __hip_atomic_load(shares + ep_rank * a.sh.D + d, __ATOMIC_RELAXED,
@@ -332,17 +376,31 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
       __builtin_amdgcn_s_sleep(2);
     if (polls >= kMaxPolls)
       __hip_atomic_fetch_add(a.sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    set_replica(table, replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local],
-                __builtin_bit_cast(float, (uint32_t)word), a.o2r[(ep_rank % a.sh.G) * a.sh.D + d]);
+    return __builtin_bit_cast(float, (uint32_t)word);
+  };
+  if (set0) {
+    const float share = share_of(rank0, local0 % a.sh.D);
+    if (le0 >= 0)
+      table[le0].expected = expected_on_original(share, total0);
+  }
+  for (int i = tid + nt; i < n_sets; i += nt) {
+    const int ep_rank = i / cd, local = i % cd;
+    const float share = share_of(ep_rank, local % a.sh.D);
+    const int le = a.phy2log[ep_rank * a.sh.P + local];
+    if (le >= 0 && le < nl)
+      table[le].expected = expected_on_original(share, table[le].total);
   }
   __syncthreads();
 #pragma unroll
   for (int c = 0; c < K; ++c) {
-    const int64_t o = redirect_token<false>(ev[c], mine, table, replica, my_bit);
+    int64_t o = -1;
+    if (ev[c] >= 0) {
+      const ExpertEntry x = table[ev[c]];
+      o = h[c] >= x.expected ? replica[ev[c]] : x.original;
+    }
     const int64_t i = begin + ((int64_t)wave * K + c) * kWave + lane;
     if (i < end)
       __builtin_nontemporal_store(o, a.out + i);
-    __builtin_amdgcn_wave_barrier();
   }
   if (pid == 0 && a.physical_counts)
     emit_physical_counts(table, replica, a.sh, a.phy2log, a.physical_counts, tid, nt);
