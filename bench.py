@@ -34,7 +34,7 @@ REDIRECT_BYTES_PER_INDEX = 16
 # HBM bytes one redirect launch moves at the sweep shape, from rocprofv3 FETCH_SIZE and WRITE_SIZE (two
 # runs), each scaled by what the same counter reads for the plain copy kernel of known size:
 # 16 797 KiB read + 16 376 KiB written, 1.012 x the algorithmic bytes.
-REDIRECT_TRAFFIC_BYTES_SWEEP = 34_238_000
+REDIRECT_TRAFFIC_BYTES_SWEEP = 34_341_000
 HISTOGRAM_BYTES_PER_INDEX = 8
 
 
