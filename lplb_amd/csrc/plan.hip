@@ -601,6 +601,9 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
   LPLB_REQUIRE(step_rule == LPLB_STEP_REFERENCE_WINDOW || step_rule == LPLB_STEP_FULL_MAX, LPLB_EINVAL,
                "plan: unknown step_rule %d", step_rule);
   LPLB_REQUIRE(n_steps >= 0, LPLB_EINVAL, "plan: n_steps=%d", n_steps);
+  // refused before anything is enqueued, not by the last of the chain's kernels
+  LPLB_REQUIRE(!(physical_counts && n_elements > (INT32_MAX - 41) / 499), LPLB_EUNSUPPORTED,
+               "plan: physical_counts needs n_elements <= %d", (INT32_MAX - 41) / 499);
   const int n_logical = n_group * group_size * L;
   hipStream_t s = static_cast<hipStream_t>(stream);
   bool done = false;

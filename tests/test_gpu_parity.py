@@ -513,6 +513,42 @@ def test_redirect_full_size_sweep(cuda):
             assert phys[rank * shape.P + slot] == keep, (rank, slot)
 
 
+@pytest.mark.gpu
+def test_redirect_when_the_hash_wraps(cuda):
+    """An expert with more than (2^31 - 42) / 499 = 4 303 556 tokens makes 499 k + 41 wrap to negative
+    int32 values, whose remainder is negative too (minilp.cu:505 computes in int).  Bit-exact against
+    the oracle, through both the three entry points and the single call."""
+    c = synth.CONFIGS["cpu_ref_ep8"]
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    phy2log = planner.phy2log.cpu().numpy()
+    rng = np.random.default_rng(4303557)
+    n = 12_000_000
+    heavy = int(phy2log.reshape(c.ep_size, shape.P)[3, 0])      # an expert that has a replica
+    p = np.full(c.n_logical, 0.45 / (c.n_logical - 1))
+    p[heavy] = 0.55
+    idx = rng.choice(c.n_logical, size=n, p=p).astype(np.int64)
+    idx[rng.random(n) < 0.01] = -1
+    assert np.count_nonzero(idx == heavy) > 6_000_000
+    d_idx = dev(idx, cuda)
+    n_sms = 256
+    local, by_sm = planner.count_workload(d_idx, n_sms)
+    want_by_sm = oracle.count_idx(idx, c.n_logical, n_sms)
+    np.testing.assert_array_equal(by_sm.cpu().numpy(), want_by_sm)
+    o_weight, _ = planner.solve_probs(local, torch.zeros(1, dtype=torch.int32, device=cuda))
+    got = planner.weighted_select_target(d_idx, o_weight, by_sm, n_sms).cpu().numpy()
+    want = oracle.map_idx(idx, o_weight.cpu().numpy(), want_by_sm, shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
+    np.testing.assert_array_equal(got, want)
+    both = np.unique(got[idx == heavy])
+    assert len(both) == 2                                        # the heavy expert really is split
+    out = planner.run(d_idx, torch.zeros(1, dtype=torch.int32, device=cuda), n_sms)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+    # the closed form behind physical_counts assumes no wrap: asked for here, it is refused
+    with pytest.raises(RuntimeError, match="physical_counts"):
+        planner.run(d_idx, torch.zeros(1, dtype=torch.int32, device=cuda), n_sms,
+                    physical_counts=torch.empty(c.n_physical, dtype=torch.int32, device=cuda))
+
+
 # ------------------------------------------------------- single-call plan, graphs
 def _plan_setup(cuda, cfg_name, mask=0.05):
     inp = synth.make_inputs(cfg_name, mask_fraction=mask)

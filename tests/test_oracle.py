@@ -112,6 +112,35 @@ def test_redirect_matches_definition_on_small_inputs(seed):
         np.testing.assert_array_equal(got, want)
 
 
+def test_redirect_hash_wraps_like_32_bit_int_arithmetic():
+    """minilp.cu:505 computes (k * 499 + 41) % total in int: beyond k = 4 303 556 the product wraps to
+    negative values and the remainder takes the sign of the dividend.  Restated here in 64-bit
+    arithmetic with the wrap and the truncating remainder written out."""
+    r2o, ep, nl = np.asarray(topology.RING_8P), 8, 16
+    phy2log, _, _ = build_redundancy_mapping(r2o, ep, nl, nl + ep, None)
+    s = Shape(r2o, ep, nl, nl + ep)
+    heavy = int(np.asarray(phy2log).reshape(ep, s.P)[2, 0])        # has a replica
+    n = 5_000_000
+    idx = np.full(n, heavy, np.int64)
+    idx[::1000] = (heavy + 1) % nl
+    w = np.full((1, s.G, s.D), 0.4, np.float32)
+    by_sm = oracle.count_idx(idx, nl, 64)
+    got = oracle.map_idx(idx, w, by_sm, s.o2r, phy2log, 1, s.C, s.P)
+    mine = idx == heavy
+    total = int(mine.sum())
+    assert total > 4_303_557
+    k = np.arange(total, dtype=np.int64)
+    h = (k * 499 + 41 + 2 ** 31) % 2 ** 32 - 2 ** 31             # what a 32-bit int holds
+    assert h.min() < 0
+    rem = np.fmod(h, total)                                       # truncating, sign of the dividend
+    expected = int(np.trunc(np.float32(0.4) * np.float32(total)))
+    slots = np.unique(got[mine])
+    assert len(slots) == 2
+    original = 2 * s.P
+    replica = int(slots[slots != original][0])
+    np.testing.assert_array_equal(got[mine], np.where(rem < expected, original, replica))
+
+
 def test_redirect_reference_test_properties():
     """tests/test_idx_processing.py:51-138 of the reference, on a numpy draw."""
     name, r2o, nl, ep, red, _, _ = REFERENCE_SOLVE_CASES[0]
