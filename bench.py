@@ -347,6 +347,20 @@ def main() -> None:
         def plan_local():
             assert lib.lplb_plan(*local_args, stream) == 0
         extras["plan_local_counts_us_p50"] = round(pct(event_times_us(plan_local, 1000, 100, torch), 50), 2)
+        # the same plan on inputs that are not in any cache: 320 distinct index / output pairs
+        # (1 MiB each, together more than the 256 MB the last-level cache holds), used in turn
+        n_cold = 320
+        cold_idx = torch.stack([torch.roll(idx.reshape(-1), 131 * i) for i in range(n_cold)])
+        cold_out = torch.empty_like(cold_idx)
+        cold_args = [(cold_idx[i].data_ptr(),) + plan_args[1:16] + (cold_out[i].data_ptr(),) + plan_args[17:]
+                     for i in range(n_cold)]
+        turn = [0]
+
+        def plan_cold():
+            turn[0] = (turn[0] + 1) % n_cold
+            assert lib.lplb_plan(*cold_args[turn[0]], stream) == 0
+        extras["plan_inputs_from_hbm_us_p50"] = round(pct(event_times_us(plan_cold, 1280, 320, torch), 50), 2)
+        del cold_idx, cold_out
         assert lib.lplb_plan_set_cooperative(0) == 0
         extras["plan_as_chain_us_p50"] = round(pct(event_times_us(plan, 1000, 100, torch), 50), 2)
         extras["plan_local_counts_as_chain_us_p50"] = round(pct(event_times_us(plan_local, 1000, 100, torch), 50), 2)
