@@ -211,7 +211,7 @@ int lplb_plan_set_cooperative(int enabled);
  * for each other with a bounded number of polls; *count receives how many waits
  * ran out on the current device since the library was loaded (0 in a healthy
  * run; a plan with a wait that ran out has undefined output).  Synchronous:
- * copies one int from the device.
+ * copies a few ints from the device.
  */
 int lplb_plan_sync_timeouts(int *count);
 
