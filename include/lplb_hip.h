@@ -162,7 +162,7 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  * One batch's whole plan in a single call: what Planner.run does with three
  * extension calls (lplb/planner.py:245-266), with the same results as
  * lplb_count_idx, lplb_solve and lplb_map_idx chained on `stream`.  Short
- * batches (up to 262144 indices) of LP shapes up to 32 x 2 run as ONE kernel launch in
+ * batches (up to 262144 indices) of LP shapes up to 32 x 2 and up to 32 EP groups run as ONE kernel launch in
  * which the workgroups exchange their histogram rows and the LP's result through
  * memory; everything else runs as the chain of the three entry points' kernels.
  *
@@ -184,7 +184,7 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  * block for each of the first eight streams that plan (further streams get the
  * chain).  Launches that share a block must not overlap in time, which stream order
  * guarantees; the exception is a graph captured on one stream and replayed
- * concurrently on several.  A launch takes up to a quarter of the GPU's CUs and its
+ * concurrently on several.  A launch takes up to a quarter of the GPU's CUs (plus one per four EP groups) and its
  * workgroups wait for each other, so at most three plans may execute at the same
  * time on a device (see lplb_plan_set_cooperative).
  */

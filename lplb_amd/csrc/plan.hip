@@ -14,7 +14,7 @@
 // or 1024-thread workgroup.  Every
 // kernel boundary of the chain costs 3-5 us on this GPU although the kernels have
 // 1-3 us of work, and the LP (8 us, one wave) sits on the critical path.  Here one
-// workgroup per slice and one more for the LP run side by side in a single grid:
+// workgroup per slice and one more per four LPs run side by side in a single grid:
 //   slice workgroup: load indices -> per-wave LDS histograms -> publish the slice's
 //     histogram row -> wait until all rows are there -> add up the rows (totals and
 //     counts before this slice) -> tables and per-wave starting ordinals -> wait for
@@ -24,7 +24,7 @@
 // What crosses workgroups (rows, shares, three counters) is written and read with
 // agent-scope atomics, which go through the XCD's L2 to memory; nothing else is
 // shared, so no cache write-back or invalidate is needed.  The grid is far smaller
-// than the GPU (at most 65 workgroups on 256 CUs), so all workgroups are resident
+// than the GPU (at most 72 workgroups on 256 CUs), so all workgroups are resident
 // and the waits end; each wait is bounded all the same, and a wait that runs out is
 // counted (lplb_plan_sync_timeouts) instead of hanging the GPU.  The counters live
 // in a per-device array of this library, one block per stream (the first eight streams
@@ -45,6 +45,11 @@ constexpr int kMaxSlices = 64;         // slice workgroups of the one-launch pla
 constexpr int kChunksPerWave = 4;     // its longest slice: 4 chunks of 64 indices per wave
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
 constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait gives up
+// LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP
+// wave is bound by instruction issue, so a fifth LP on the same CU would slow two of them
+// down (8 LPs in one workgroup: 17.0 us per plan against 13.5 us).  Batches with more
+// groups get more LP workgroups.
+constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 
 // [0] slices whose histogram row is published, [1] workgroups that have left,
 // [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
@@ -53,11 +58,11 @@ constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait 
 // batch's tokens of that expert in the high half and the number of slices that have
 // added theirs in the low half -- one atomic add per slice and expert delivers both,
 // so the reader needs no second round trip for a "done" counter.
-constexpr int kSharesAt = 16, kMaxShares = 256;
+constexpr int kSharesAt = 16, kMaxShares = 1024;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
 // One such block per stream that has run a plan (the compute stream, a warm-up
 // stream, a graph-capture stream ...), so that plans enqueued on different streams
-// do not share counters.  A launch takes at most a quarter of the CUs: up to three
+// do not share counters.  A launch takes at most a quarter of the CUs (+ 8): up to three
 // plans that really execute at the same time are all resident; with four or more,
 // workgroups could wait for workgroups that cannot start.
 constexpr int kSlotInts = kTotalsAt + 2 * kMaxTotals, kSyncSlots = 8;
@@ -67,7 +72,7 @@ static std::atomic<bool> g_cooperative{true};   // any thread may flip it while 
 struct PlanArgs {
   const int64_t *idx;
   int64_t n, per;
-  int n_slices;
+  int n_slices, n_lp_workgroups;
   const int32_t *o2r, *phy2log;
   int32_t *rows;     // [n_slices][n_logical] per-slice histograms, exchanged between workgroups
   int32_t *totals;   // [n_logical] this GPU's tokens per expert, out
@@ -165,13 +170,15 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
   const int lane = tid % kWave, wave = tid / kWave;
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, but known to be wave-uniform
   const int pid = blockIdx.x;
-  const int n_workgroups = a.n_slices + 1;
+  const int n_workgroups = a.n_slices + a.n_lp_workgroups;
   const int n_shares = a.sh.n_ranks * a.sh.D;
   const int n_groups = nt >= nl ? nt / nl : 1;   // threads per expert when rows are added up
 
-  if (pid == a.n_slices) {
-    // ------------------------------------------------------------ the LP
+  if (pid >= a.n_slices) {
+    // ------------------------------------------------------------ the LPs
     SolveArgs sa = a.solve;
+    const int first_lp = (pid - a.n_slices) * kLpsPerWorkgroup;          // of this workgroup
+    const int n_lps = min(kLpsPerWorkgroup, sa.n_units - first_lp);
     LPLB_PLAN_STAMP(0);
     // Own-histogram mode: the LP waves start at once (their table loads do not need
     // the counts) and pick the counts up from LDS; the wave after them waits for the
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
         counts_ready = 0;
       __syncthreads();
       sa.counts_ready = &counts_ready;
-      if (wave == sa.n_units) {
+      if (wave == n_lps) {
         // Poll the totals until every expert's word says that all slices have added
         // theirs (plain loads after an acquire fence: they can be batched).
         const unsigned long long *words = reinterpret_cast<const unsigned long long *>(a.sync + kTotalsAt);
@@ -211,18 +218,19 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
           }
           __builtin_amdgcn_s_sleep(2);
         }
-        for (int e = lane; e < nl; e += kWave)   // this GPU's totals, for the caller
-          a.totals[e] = (int32_t)staged[e];
+        if (pid == a.n_slices)
+          for (int e = lane; e < nl; e += kWave)   // this GPU's totals, for the caller
+            a.totals[e] = (int32_t)staged[e];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
           __hip_atomic_store(&counts_ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
     }
     LPLB_PLAN_STAMP(1);
-    if (wave < sa.n_units) {
+    if (wave < n_lps) {
       // (own-histogram mode: every LP of the batch reads the one staged copy)
       float *mine = a.local_counts ? staged : staged + (size_t)wave * sa.staged_stride;
-      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, wave, mine, rep_of_edge_all + wave * kWave);
+      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, first_lp + wave, mine, rep_of_edge_all + wave * kWave);
       if (lane == 0 && n_ok > 0)
         atomicAdd(sa.avail, n_ok);
     }
@@ -415,7 +423,7 @@ static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t
     if (err != hipSuccess)
       return err;
   }
-  launch(plan_in_one_launch<GM, DM, EXACT, K, WAVES>, dim3(a.n_slices + 1), dim3(WAVES * kWave), lds, s, a);
+  launch(plan_in_one_launch<GM, DM, EXACT, K, WAVES>, dim3(a.n_slices + a.n_lp_workgroups), dim3(WAVES * kWave), lds, s, a);
   return hipGetLastError();
 }
 
@@ -439,7 +447,7 @@ template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanAr
   const int64_t chunks = (a.per + kWave - 1) / kWave;
   const int k = (int)((chunks + W - 1) / W);
   const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, W);
-  const size_t lds_lp = (size_t)a.solve.n_units * a.solve.n_experts * sizeof(float);
+  const size_t lds_lp = (size_t)min(a.solve.n_units, kLpsPerWorkgroup) * a.solve.n_experts * sizeof(float);
   a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
   if (a.local_counts && a.solve.staged_stride == 0)   // the LP takes its counts from LDS in that mode
     return hipErrorInvalidValue;
@@ -496,11 +504,13 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (!g_cooperative || n_elements <= 0 || n_blocks < 2)
     return LPLB_OK;
   int gm = 0, dm = 0;
-  if (!plan_lp_shape(G, D, &gm, &dm) || n_group > 8 || n_group * G * D > kMaxShares || global_workload == nullptr)
+  if (!plan_lp_shape(G, D, &gm, &dm) || n_group > kLpsPerWorkgroup * kMaxLpWorkgroups ||
+      n_group * G * D > kMaxShares || global_workload == nullptr)
     return LPLB_OK;
   const int waves = plan_waves(gm, dm);
-  // own-histogram mode: a spare wave beside the LPs, the totals fit the accumulator and the LDS
-  if (counts == nullptr && (n_group >= waves || n_logical > kMaxTotals))
+  const int n_lp_workgroups = (n_group + kLpsPerWorkgroup - 1) / kLpsPerWorkgroup;
+  // own-histogram mode: the totals fit the accumulator (and with it the LDS)
+  if (counts == nullptr && n_logical > kMaxTotals)
     return LPLB_OK;
   // slices of 1024 indices while kMaxSlices of them cover the batch, else of 2048, else of
   // 4096; at most n_blocks - 1 of them (the caller's bound on parallelism; the last row of
@@ -520,12 +530,13 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (rc != LPLB_OK)
     return rc;
   const int slot = sync_slot_of(s);
-  if (slices + 1 > n_cus / 4 + 1 || slot < 0)
+  // a quarter of the CUs for the slices, so that three plans that execute at once are all resident
+  if (slices > n_cus / 4 || slot < 0)
     return LPLB_OK;
   sync += (size_t)slot * kSlotInts;
 
   PlanArgs a{};   // every field the host does not set below is zero
-  a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices;
+  a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices; a.n_lp_workgroups = n_lp_workgroups;
   a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block;
   a.totals = counts_by_block + (int64_t)(n_blocks - 1) * n_logical; a.out = out;
   a.physical_counts = physical_counts;

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from lplb_amd import Planner, synth
+from lplb_amd import Planner, synth, topology
 from lplb_amd._native import CompiledSolver
 from oracle import oracle
 from tests.helpers import CASE_SEED, REFERENCE_SOLVE_CASES, Shape, reference_style_case
@@ -589,8 +589,43 @@ def test_plan_entry_point_matches_three_calls(cuda, cfg, use_global):
 def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
     """Short batches run as one kernel launch whose workgroups exchange histogram rows and the
     LP's shares through memory; the result must be the chain's, bit for bit, call after call."""
-    from lplb_amd import _native
     inp = synth.make_inputs(cfg, tokens=tokens, mask_fraction=0.05) if tokens else synth.make_inputs(cfg, mask_fraction=0.05)
+    _one_launch_equals_chain(cuda, inp, use_global, n_sms)
+
+
+MANY_GROUPS = {
+    # the LPs of a batch are spread over workgroups of four: 5 groups leave the second one partly empty
+    "ep40_5_cubes": synth.PlanConfig("ep40", topology.CUBE_8P2E, 40, 240, 2, 4096, 8, 1.0, jitter_sigma=0.3, seed=40),
+    "v3_ep64_8_cubes": synth.PlanConfig("ep64", topology.CUBE_8P2E, 64, 256, 2, 4096, 8, 1.0, jitter_sigma=0.3, seed=64),
+    "v3_ep128_16_cubes": synth.PlanConfig("ep128", topology.CUBE_8P2E, 128, 256, 2, 512, 8, 1.0, jitter_sigma=0.3, seed=128),
+    "v3_ep256_32_rings": synth.PlanConfig("ep256", topology.RING_8P, 256, 256, 1, 128, 8, 1.0, jitter_sigma=0.3, seed=256),
+    "v3_ep64_4_hypercubes": synth.PlanConfig("ep64h", topology.HYPERCUBE_16P2E, 64, 256, 2, 4096, 8, 1.0, seed=65),
+    "v3_ep192_6_tori": synth.PlanConfig("ep192", topology.torus_2d(8, 4), 192, 384, 2, 2048, 8, 1.0, seed=192),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(MANY_GROUPS))
+@pytest.mark.parametrize("use_global", [True, False])
+def test_plan_one_launch_with_many_groups(cuda, name, use_global):
+    """Large EP sizes: several LPs per batch, up to four per LP workgroup."""
+    inp = synth.make_inputs(MANY_GROUPS[name], mask_fraction=0.02)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    got = _one_launch_equals_chain(cuda, inp, use_global, 256)
+    # and the chain's result is the oracle's
+    counts = inp.global_counts if use_global else np.bincount(inp.indices[inp.indices >= 0].ravel(),
+                                                              minlength=c.n_logical).astype(np.int32)
+    _, _, o_avail = oracle.solve(counts, shape.r2o, inp.phy2log, shape.n_group, shape.C, shape.n_fixed)
+    assert got[3] == o_avail
+    by_sm = oracle.count_idx(inp.indices.reshape(-1), c.n_logical, 256)
+    want = oracle.map_idx(inp.indices.reshape(-1), got[1], by_sm, shape.o2r, inp.phy2log, shape.n_group, shape.C,
+                          shape.P).reshape(inp.indices.shape)
+    np.testing.assert_array_equal(got[0], want)
+
+
+def _one_launch_equals_chain(cuda, inp, use_global, n_sms):
+    from lplb_amd import _native
     c = inp.cfg
     shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
     solver = solver_for(shape)
@@ -619,6 +654,7 @@ def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
                                                              minlength=c.n_logical))
     out = runs[True][0]
     np.testing.assert_array_equal(runs[True][4], np.bincount(out[out >= 0].ravel(), minlength=c.n_physical))
+    return runs[True]
 
 
 def test_plan_random_shapes_one_launch_equals_chain(cuda):
@@ -629,7 +665,8 @@ def test_plan_random_shapes_one_launch_equals_chain(cuda):
     rng = np.random.default_rng(77)
     topologies = [(topology.CUBE_8P2E, 1), (topology.RING_8P, 1), (topology.HYPERCUBE_16P2E, 1),
                   (topology.torus_2d(8, 4), 1), (topology.CUBE_8P2E, 4), (_shifted_ring(6, [1, 2]), 2),
-                  (_shifted_ring(4, [1, 2, 3]), 3), (_shifted_ring(16, [1]), 2)]
+                  (_shifted_ring(4, [1, 2, 3]), 3), (_shifted_ring(16, [1]), 2), (topology.CUBE_8P2E, 9),
+                  (topology.RING_8P, 16)]
     try:
         for trial in range(30):
             r2o, n_group = topologies[int(rng.integers(len(topologies)))]
