@@ -162,7 +162,7 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  * One batch's whole plan in a single call: what Planner.run does with three
  * extension calls (lplb/planner.py:245-266), with the same results as
  * lplb_count_idx, lplb_solve and lplb_map_idx chained on `stream`.  Short
- * batches (up to 262144 indices) of LP shapes up to 32 x 2 and up to 32 EP groups run as ONE kernel launch in
+ * batches (up to 524288 indices) of LP shapes up to 32 x 2 and up to 32 EP groups run as ONE kernel launch in
  * which the workgroups exchange their histogram rows and the LP's result through
  * memory; everything else runs as the chain of the three entry points' kernels.
  *

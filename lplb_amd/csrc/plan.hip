@@ -9,8 +9,8 @@
 // as a parallel branch of a captured HIP graph (side stream + events) was measured
 // and rejected: 24.6 us per plan against 20.0 us for the plain chain in the graph.
 //
-// One launch (plan_in_one_launch): for batches of up to 64 slices of 4096 indices
-// (2048 with 512-thread workgroups) and LP shapes whose registers fit beside a 512-
+// One launch (plan_in_one_launch): for batches of up to 64 slices of 8192 indices
+// (4096 with 512-thread workgroups) and LP shapes whose registers fit beside a 512-
 // or 1024-thread workgroup.  Every
 // kernel boundary of the chain costs 3-5 us on this GPU although the kernels have
 // 1-3 us of work, and the LP (8 us, one wave) sits on the critical path.  Here one
@@ -42,7 +42,7 @@
 namespace lplb {
 
 constexpr int kMaxSlices = 64;         // slice workgroups of the one-launch plan
-constexpr int kChunksPerWave = 4;     // its longest slice: 4 chunks of 64 indices per wave
+constexpr int kChunksPerWave = 8;     // its longest slice: 8 chunks of 64 indices per wave
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
 constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait gives up
 // LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP
@@ -455,7 +455,9 @@ template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanAr
     return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s);
   if (k <= 2)
     return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds_slices, s);
-  return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s);
+  if (k <= 4)
+    return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s);
+  return launch_plan_variant<GM, DM, EXACT, 8, W>(a, lds_slices, s);
 }
 
 // The block of counters a stream uses: the first kSyncSlots streams that run a plan
@@ -512,8 +514,8 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   // own-histogram mode: the totals fit the accumulator (and with it the LDS)
   if (counts == nullptr && n_logical > kMaxTotals)
     return LPLB_OK;
-  // slices of 1024 indices while kMaxSlices of them cover the batch, else of 2048, else of
-  // 4096; at most n_blocks - 1 of them (the caller's bound on parallelism; the last row of
+  // slices of 1024 indices while kMaxSlices of them cover the batch, else of 2048, 4096,
+  // 8192; at most n_blocks - 1 of them (the caller's bound on parallelism; the last row of
   // its table takes the totals)
   int64_t slices = kMaxSlices + 1;
   for (int64_t len = 1024; len <= (int64_t)waves * kChunksPerWave * kWave && slices > kMaxSlices; len *= 2)
