@@ -298,6 +298,53 @@ def test_solve_adversarial_distributions(cuda, topo):
     assert flags_differ <= 2 and checked >= 40
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("G,D,C,n_group", [(3, 1, 1, 1), (5, 2, 1, 3), (6, 3, 2, 1), (7, 4, 1, 2), (8, 8, 1, 1),
+                                           (10, 6, 1, 1), (12, 2, 3, 2), (12, 5, 1, 1), (16, 4, 1, 1), (21, 3, 1, 1),
+                                           (24, 2, 1, 2), (32, 2, 2, 1), (40, 1, 1, 1), (64, 1, 1, 1)])
+def test_solve_random_topologies(cuda, G, D, C, n_group):
+    """Replica topologies that are no named graph: every column of r2o is a random permutation
+    (self-loops included), group sizes that do not fill the kernels' register arrays (padded
+    instantiations), several replicated experts per slot.  Yardstick: the fp64 oracle."""
+    rng = np.random.default_rng(1000 * G + 10 * D + C)
+    r2o = np.stack([rng.permutation(G) for _ in range(D)], axis=1).astype(np.int32)
+    ep = G * n_group
+    per_rank = D * C + int(rng.integers(0, 5))
+    nl = ep * per_rank
+    shape = Shape(r2o, ep, nl, nl + D * C * ep)
+    assert (shape.C, shape.n_fixed) == (C, per_rank - D * C)
+    solver = solver_for(shape)
+    compared = 0
+    for trial in range(6):
+        # any assignment of logical experts to slots is a legal phy2log layout: originals are a
+        # permutation, replica slot (rank, c*D+d) copies slot c*D+d of rank r2o[rank][d]
+        originals = rng.permutation(nl).reshape(ep, per_rank)
+        phy2log = np.empty((ep, shape.P), np.int32)
+        phy2log[:, :per_rank] = originals
+        for rank in range(ep):
+            g0 = rank // G * G
+            for c in range(C):
+                for d in range(D):
+                    phy2log[rank, per_rank + c * D + d] = originals[g0 + r2o[rank % G, d], c * D + d]
+        phy2log = phy2log.reshape(-1)
+        p = rng.dirichlet(np.full(nl, [0.3, 1.0, 5.0][trial % 3]))
+        wl = rng.multinomial(int(rng.choice([2000, 1 << 17, 1 << 22])), p).astype(np.int32)
+        wl[rng.integers(nl)] += 1          # never all zero
+        avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+        res, gw = solver.solve(dev(wl.reshape(n_group, G, per_rank), cuda), dev(r2o, cuda), dev(phy2log, cuda), avail)
+        res = res.cpu().numpy()
+        o64, o_gw, o_avail = oracle.solve(wl, r2o, phy2log, n_group, C, shape.n_fixed, precision=64)
+        np.testing.assert_array_equal(gw.cpu().numpy().reshape(-1), o_gw)
+        if int(avail[0]) != o_avail or o_avail != n_group:
+            continue                        # a flag on the edge of a threshold; counted below
+        args = (r2o, phy2log, n_group, C)
+        flow = np.abs(oracle.edge_flows(wl, res, *args) - oracle.edge_flows(wl, o64, *args)).max() / float(wl.sum())
+        obj, obj64 = (oracle.rank_loads(wl, x, *args).max(axis=1) for x in (res, o64))
+        assert flow <= FLOW_TOL and float((np.abs(obj - obj64) / obj64).max()) <= OBJ_RTOL, (trial, flow)
+        compared += 1
+    assert compared >= 4
+
+
 def test_solve_fallback_and_counter(cuda):
     """Infeasible / degenerate LPs give 0.5 everywhere and leave the counter alone;
     the counter accumulates across calls (minilp.cu:379-400)."""
