@@ -8,7 +8,7 @@ namespace lplb {
 // Per-expert constants of the redirect, one 16-byte LDS read per token.
 struct __attribute__((aligned(16))) ExpertEntry {
   int32_t total;     // tokens of this expert in the whole index array
-  uint32_t magic;    // floor(2^32 / total) (all ones for total == 1, 0 for total <= 0)
+  uint32_t magic;    // floor((2^32 - 1) / total), 0 for total <= 0
   int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
   int32_t original;  // physical slot of the original
 };
@@ -20,8 +20,12 @@ struct __attribute__((aligned(16))) WaveSlot {
   unsigned long long bits;  // lanes of the current chunk that hold this expert
 };
 
-// h mod total with C's truncating sign rule; q = mulhi(|h|, magic) is the true
-// quotient or one less.  WRAP: the hash 499 k + 41 may have wrapped to negative.
+// h mod total with C's truncating sign rule.  magic = floor((2^32 - 1) / total) is at
+// least 2^32 / total - 1, so for a <= 2^31: a / total >= a * magic / 2^32 >=
+// a / total - 1/2.  q = mulhi(a, magic) is therefore the true quotient or one less,
+// and one conditional subtract finishes (a 32-bit division per expert instead of one
+// per token).
+// WRAP: the hash 499 k + 41 may have wrapped to negative.
 template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
   const uint32_t a = WRAP ? (uint32_t)max(h, -h) : (uint32_t)h;
   uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
@@ -45,7 +49,7 @@ __device__ inline void init_entry(ExpertEntry *table, int32_t *replica, int32_t 
                                   int32_t start) {
   ExpertEntry x;
   x.total = t;
-  x.magic = t > 1 ? (uint32_t)(0x100000000ull / (uint32_t)t) : (t == 1 ? 0xffffffffu : 0u);
+  x.magic = t >= 1 ? 0xffffffffu / (uint32_t)t : 0u;
   x.expected = t;
   x.original = -1;
   table[e] = x;
