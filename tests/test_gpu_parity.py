@@ -340,7 +340,7 @@ def test_solve_random_topologies(cuda, G, D, C, n_group):
         args = (r2o, phy2log, n_group, C)
         flow = np.abs(oracle.edge_flows(wl, res, *args) - oracle.edge_flows(wl, o64, *args)).max() / float(wl.sum())
         obj, obj64 = (oracle.rank_loads(wl, x, *args).max(axis=1) for x in (res, o64))
-        assert flow <= FLOW_TOL and float((np.abs(obj - obj64) / obj64).max()) <= OBJ_RTOL, (trial, flow)
+        assert flow <= FLOW_TOL and np.all(np.abs(obj - obj64) <= OBJ_RTOL * obj64), (trial, flow)   # a group may be empty
         compared += 1
     assert compared >= 4
 
