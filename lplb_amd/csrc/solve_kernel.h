@@ -404,9 +404,13 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // of row c through LDS instead of v_readlane halves their instruction count at
     // 32 ranks, but puts an LDS write -> read round trip into every step of the chain:
     // measured 45 us against 34 us.)
+    // A lane's own multiple must be zero.  Rather than selecting on the chain (f is the
+    // link between reciprocal and update), the lane's diagonal entry is cleared as soon
+    // as it has been read as the pivot, one step ahead.
     double my_pivot = 1.0;
     double pivot = lp_bcast<ROWS, 0>(S[0]);
     double rinv = rcp_f64(pivot);
+    S[0] = (lane == 0) ? 0.0 : S[0];
     static_for<GM>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
       auto clear = [&](auto c2c, double f) {
@@ -415,12 +419,13 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
           S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
       };
       my_pivot = (lane == c) ? pivot : my_pivot;
-      const double f = (lane != c) ? S[c] * rinv : 0.0;   // multiple of row c to subtract from my row
+      const double f = S[c] * rinv;   // multiple of row c to subtract from my row (0 in lane c)
       double next_pivot = 1.0, estimate = 1.0, error = 0.0;
       clear(std::integral_constant<int, c + 1>{}, f);
       if constexpr (c + 1 < GM) {
         next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
         estimate = __builtin_amdgcn_rcp(next_pivot);
+        S[c + 1] = (lane == c + 1) ? 0.0 : S[c + 1];
       }
       rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
       clear(std::integral_constant<int, c + 2>{}, f);
