@@ -336,6 +336,13 @@ def main() -> None:
 
         # the plan kernel's own duration, the plan fed by this GPU's own histogram (what Planner.run
         # does without a process group), and the plan as the chain of the three entry points' kernels
+        # the same plans without an event between them: wall clock of a run of 2000, one sync at the end
+        torch.cuda.synchronize()
+        t_run = time.perf_counter()
+        for _ in range(2000):
+            plan()
+        torch.cuda.synchronize()
+        extras["plan_back_to_back_wall_us"] = round((time.perf_counter() - t_run) / 2000 * 1e6, 2)
         plan_timer = KernelTimer(lib, 300)
         for _ in range(300):
             plan_timer.arm()
