@@ -213,3 +213,11 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.lplb_map_idx(p, p, p, p, None, 4, 1, 8, 2, 1, 34, 4, p, None, None) == 1
     assert lib.lplb_plan(p, 4, None, p, p, p, 1, 8, 2, 1, 34, 0, p, p, p, p, p, None, 0, 5, None) == 1
     assert lib.lplb_copy_calibration(p, p, 3, None) == 1
+    # an index array needs its natural alignment only; 4 bytes off is refused
+    odd = ctypes.c_void_p(p.value + 4)
+    assert lib.lplb_count_idx(odd, 4, 8, 4, p, None) == 1 and b"8-byte" in lib.lplb_last_error()
+    assert lib.lplb_plan(odd, 4, None, p, p, p, 1, 8, 2, 1, 34, 4, p, p, p, p, p, None, 0, 5, None) == 1
+    # tokens per physical expert come from a closed form that assumes 499 k + 41 does not wrap
+    assert lib.lplb_plan(p, 5_000_000, None, p, p, p, 1, 8, 2, 1, 34, 256, p, p, p, p, p, p, 0, 5, None) == 2
+    assert b"physical_counts" in lib.lplb_last_error()
+    assert lib.lplb_map_idx(p, p, p, p, p, 5_000_000, 1, 8, 2, 1, 34, 256, p, p, None) == 2
