@@ -403,7 +403,11 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // the compiler keeps the order it is given here.  (Broadcasting the far columns
     // of row c through LDS instead of v_readlane halves their instruction count at
     // 32 ranks, but puts an LDS write -> read round trip into every step of the chain:
-    // measured 45 us against 34 us.)
+    // measured 45 us against 34 us.  Computing the next pivot one step ahead from three
+    // more broadcasts, in uniform arithmetic, gives bit-identical results and takes the
+    // vector update out of the chain, but costs 9 instructions per pivot and was slower
+    // at 8 ranks, 7.8 us against 7.6 us: at 4.7 clocks per instruction the sweep is
+    // bound by instruction issue more than by the chain.)
     // A lane's own multiple must be zero.  Rather than selecting on the chain (f is the
     // link between reciprocal and update), the lane's diagonal entry is cleared as soon
     // as it has been read as the pivot, one step ahead.
