@@ -12,7 +12,7 @@ import functools
 import numpy as np
 import torch
 
-from ._native import CompiledSolver
+from ._native import CompiledSolver, _stream
 from .mapping import build_redundancy_mapping
 
 
@@ -82,6 +82,7 @@ class Planner:
         self.ep_group = group
         self.deep_ep_initialized = False
         self._solver: CompiledSolver | None = None
+        self._run_buffers: dict = {}
 
     @property
     def solver(self) -> CompiledSolver:
@@ -156,10 +157,19 @@ class Planner:
         """
         if n_sms is None:
             n_sms = torch.cuda.get_device_properties(idx.device).multi_processor_count
+        # run() hands out only the redirected indices, so the plan's other buffers (slice table,
+        # shares, normalised counts) are kept per stream and slice count instead of being
+        # allocated for every batch; work on one stream is ordered, so reuse is safe there
+        key = (_stream(idx), n_sms)
+        ws = self._run_buffers.get(key)
+        if ws is None:
+            if len(self._run_buffers) >= 16:
+                self._run_buffers.clear()
+            ws = self._run_buffers[key] = {}
         if self.ep_group is None:
             # count_workload -> solve_probs -> weighted_select_target in one library call
             out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
-                                                      physical_counts=physical_counts)
+                                                      workspace=ws, physical_counts=physical_counts)
             return out
         # With a process group the counts have to be summed over the ranks between histogram and
         # LP (lplb/planner.py:214-216); LP and redirect then run as one plan on the summed counts.
@@ -168,5 +178,6 @@ class Planner:
         if not self.deep_ep_initialized:
             torch.distributed.all_reduce(workload, group=self.ep_group)
         out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
-                                                  global_counts=workload, physical_counts=physical_counts)
+                                                  global_counts=workload, workspace=ws,
+                                                  physical_counts=physical_counts)
         return out
