@@ -123,6 +123,21 @@ template <int ROWS, int LANE, typename T> __device__ inline T lp_bcast(T v) {
   else
     return row_bcast<LANE>(v);
 }
+// `old` with lane LANE of this LP's lanes replaced by `v`, a value that is the same in
+// all of them.  One LP per wave: v sits in scalar registers and v_writelane puts it into
+// the lane (a select would first have to copy it into a vector register).
+template <int ROWS, int LANE> __device__ inline double lp_set_lane(double old, double v, int lane) {
+  if constexpr (ROWS == 1) {
+    int2 o = __builtin_bit_cast(int2, old);
+    const int2 n = __builtin_bit_cast(int2, v);
+    const int lo = __builtin_amdgcn_readfirstlane(n.x), hi = __builtin_amdgcn_readfirstlane(n.y);
+    asm("v_writelane_b32 %0, %1, %2" : "+v"(o.x) : "s"(lo), "n"(LANE));
+    asm("v_writelane_b32 %0, %1, %2" : "+v"(o.y) : "s"(hi), "n"(LANE));
+    return __builtin_bit_cast(double, o);
+  } else {
+    return lane == LANE ? v : old;
+  }
+}
 // Reductions over the first W lanes of this LP (W <= 16 when ROWS == 4).
 template <int ROWS, int W> __device__ inline float lp_sum(float v) {
   if constexpr (ROWS == 1) {
@@ -422,7 +437,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         if constexpr (c2 < GM)
           S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
       };
-      my_pivot = (lane == c) ? pivot : my_pivot;
+      my_pivot = lp_set_lane<ROWS, c>(my_pivot, pivot, lane);
       const double f = S[c] * rinv;   // multiple of row c to subtract from my row (0 in lane c)
       double next_pivot = 1.0, estimate = 1.0, error = 0.0;
       clear(std::integral_constant<int, c + 1>{}, f);
