@@ -457,7 +457,12 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         pivot = next_pivot;
       }
       static_for<(GM > c + 5 ? GM - c - 5 : 0)>([&](auto kk) {
-        clear(std::integral_constant<int, c + 5 + decltype(kk)::value>{}, f);
+        constexpr int k = decltype(kk)::value;
+        // From 32 ranks on a row's broadcasts would fill the scalar registers if the
+        // compiler hoisted them all; fence them off in groups of eight columns.
+        if constexpr (GM >= 32 && k % 8 == 0)
+          __builtin_amdgcn_sched_barrier(0);
+        clear(std::integral_constant<int, c + 5 + k>{}, f);
       });
     });
     if (step == 0) LPLB_STAMP(7);
