@@ -795,10 +795,22 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
 
 
 @pytest.mark.parametrize("use_global", [True, False])
-def test_plan_replays_from_a_hip_graph(cuda, use_global):
+@pytest.mark.parametrize("one_launch", [True, False])
+def test_plan_replays_from_a_hip_graph(cuda, use_global, one_launch):
     """Capture two plans into a graph; every replay, with eager work and synchronisation between
     replays, must reproduce the eager result and advance the counter.  (The one-launch plan keeps
-    counters in device memory that its last workgroup clears: a replay has the same arguments.)"""
+    counters in device memory that its last workgroup clears: a replay has the same arguments.
+    The chain of kernels is captured too: its histogram launch is marked as free to overtake
+    the LP before it.)"""
+    from lplb_amd import _native
+    _native.set_plan_cooperative(one_launch)
+    try:
+        _replay_plans_from_a_graph(cuda, use_global)
+    finally:
+        _native.set_plan_cooperative(True)
+
+
+def _replay_plans_from_a_graph(cuda, use_global):
     inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
     counts = t["counts"] if use_global else None
     avail = torch.zeros(1, dtype=torch.int32, device=cuda)
