@@ -850,6 +850,36 @@ def _replay_plans_from_a_graph(cuda, use_global):
         del scratch
 
 
+def test_planner_run_replays_from_a_hip_graph(cuda):
+    """Planner.run keeps its scratch buffers per stream; captured on torch's capture stream and
+    replayed, it still gives the eager result."""
+    inp = synth.make_inputs("v3_ep8_cube", mask_fraction=0.05)
+    c = inp.cfg
+    planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size)
+    planner.phy2log = dev(inp.phy2log, cuda)
+    idx = dev(inp.indices, cuda)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    eager = planner.run(idx, avail, 128).clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        planner.run(idx, avail, 128)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    before = int(avail[0])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = planner.run(idx, avail, 128)
+    for rep in range(3):
+        out.fill_(-9)
+        assert torch.equal(planner.run(idx, avail, 128), eager)     # eager calls between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        assert int(avail[0]) == before + 2 * (rep + 1)
+
+
 @pytest.mark.parametrize("cooperative", [False, True])
 def test_plans_on_two_streams(cuda, cooperative):
     """Plans on different streams may overlap on the device.  The one-launch form keeps its
