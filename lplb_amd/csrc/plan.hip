@@ -442,8 +442,7 @@ static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
   return false;
 }
 
-template <int GM, int DM, bool EXACT> static hipError_t launch_plan_shape(PlanArgs &a, hipStream_t s) {
-  constexpr int W = plan_waves(GM, DM);
+template <int GM, int DM, bool EXACT, int W> static hipError_t launch_plan_shape(PlanArgs &a, hipStream_t s) {
   const int64_t chunks = (a.per + kWave - 1) / kWave;
   const int k = (int)((chunks + W - 1) / W);
   const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, W);
@@ -509,7 +508,11 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   if (!plan_lp_shape(G, D, &gm, &dm) || n_group > kLpsPerWorkgroup * kMaxLpWorkgroups ||
       n_group * G * D > kMaxShares || global_workload == nullptr)
     return LPLB_OK;
-  const int waves = plan_waves(gm, dm);
+  // Shapes built for 16 waves also exist with 8: a slice workgroup's LDS grows with
+  // waves x logical experts, and from about 400 experts on only 8 waves fit.
+  int waves = plan_waves(gm, dm);
+  if (waves == 16 && plan_lds_bytes(n_logical, 16) > (size_t)kPlanLdsLimit)
+    waves = 8;
   const int n_lp_workgroups = (n_group + kLpsPerWorkgroup - 1) / kLpsPerWorkgroup;
   // own-histogram mode: the totals fit the accumulator (and with it the LDS)
   if (counts == nullptr && n_logical > kMaxTotals)
@@ -553,13 +556,14 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   sa.clocks = debug_clocks();
 
   hipError_t err = hipErrorInvalidValue;
-#define LPLB_PLAN_CASE(GM, DM)                                                                 \
-  if (gm == GM && dm == DM)                                                                    \
-    err = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true>(a, s)                        \
-                               : launch_plan_shape<GM, DM, false>(a, s);
-  LPLB_PLAN_CASE(8, 1) LPLB_PLAN_CASE(8, 2) LPLB_PLAN_CASE(8, 4) LPLB_PLAN_CASE(16, 1) LPLB_PLAN_CASE(16, 2)
-  LPLB_PLAN_CASE(32, 1) LPLB_PLAN_CASE(32, 2)
-#undef LPLB_PLAN_CASE
+#define LPLB_PLAN_CASE_W(GM, DM, W)                                                            \
+  if (gm == GM && dm == DM && waves == W)                                                      \
+    err = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true, W>(a, s)                     \
+                               : launch_plan_shape<GM, DM, false, W>(a, s);
+  LPLB_PLAN_CASE_W(8, 1, 16) LPLB_PLAN_CASE_W(8, 1, 8) LPLB_PLAN_CASE_W(8, 2, 16) LPLB_PLAN_CASE_W(8, 2, 8)
+  LPLB_PLAN_CASE_W(8, 4, 8) LPLB_PLAN_CASE_W(16, 1, 16) LPLB_PLAN_CASE_W(16, 1, 8) LPLB_PLAN_CASE_W(16, 2, 8)
+  LPLB_PLAN_CASE_W(32, 1, 8) LPLB_PLAN_CASE_W(32, 2, 8)
+#undef LPLB_PLAN_CASE_W
   LPLB_HIP_TRY(err);
   *done = true;
   return LPLB_OK;

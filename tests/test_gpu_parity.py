@@ -648,6 +648,10 @@ MANY_GROUPS = {
     "v3_ep256_32_rings": synth.PlanConfig("ep256", topology.RING_8P, 256, 256, 1, 128, 8, 1.0, jitter_sigma=0.3, seed=256),
     "v3_ep64_4_hypercubes": synth.PlanConfig("ep64h", topology.HYPERCUBE_16P2E, 64, 256, 2, 4096, 8, 1.0, seed=65),
     "v3_ep192_6_tori": synth.PlanConfig("ep192", topology.torus_2d(8, 4), 192, 384, 2, 2048, 8, 1.0, seed=192),
+    # more logical experts: the slice workgroups' LDS tables then leave room for 8 waves only
+    "ep8_512_experts": synth.PlanConfig("e512", topology.CUBE_8P2E, 8, 512, 2, 4096, 10, 1.0, jitter_sigma=0.3, seed=512),
+    "ep32_384_experts": synth.PlanConfig("e384", topology.CUBE_8P2E, 32, 384, 2, 4096, 8, 1.0, jitter_sigma=0.3, seed=384),
+    "ep16_1024_experts": synth.PlanConfig("e1024", topology.HYPERCUBE_16P2E, 16, 1024, 2, 2048, 8, 1.0, seed=1024),
 }
 
 
