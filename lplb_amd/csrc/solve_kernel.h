@@ -340,9 +340,19 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 #pragma unroll
   for (int u = 0; u < KB; ++u)
     part += fixed_cnt[u] / wmax;
+  // ranks with more fixed experts than were prefetched: the rest in batches of
+  // independent loads (added in the same order as one by one)
   if (br < G)
-    for (int j = bsub + KB * T; j < n_fixed; j += T)
-      part += count_of(p2l[br * P + D * C + j]) / wmax;
+    for (int j0 = bsub + KB * T; j0 < n_fixed; j0 += KB * T) {
+      int more_e[KB];
+#pragma unroll
+      for (int u = 0; u < KB; ++u)
+        more_e[u] = j0 + u * T < n_fixed ? p2l[br * P + D * C + j0 + u * T] : -1;
+#pragma unroll
+      for (int u = 0; u < KB; ++u)
+        if (j0 + u * T < n_fixed)
+          part += count_of(more_e[u]) / wmax;
+    }
   if (T >= 2) part += dpp<kQuadSwap1>(part);
   if (T >= 4) part += dpp<kQuadSwap2>(part);
   if (T >= 8) part += dpp<kHalfMirror>(part);
