@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 2
+#define LPLB_ABI_VERSION 3
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -197,6 +197,35 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
               float *global_workload, float *o_weight, int32_t *avail_num,
               int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
               lplb_stream_t stream);
+
+/*
+ * lplb_plan for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference (its extension allocates its outputs with at::empty on every call,
+ * csrc/plugin.cpp:504-505, 532-534, 586-587, 630).
+ *
+ * Same arguments, results and error codes as lplb_plan, except that the slice table
+ * (lplb_plan's counts_by_block workspace) is not passed in: it lives in a fixed
+ * 1 MiB array inside the library, one copy per GPU, held until the process ends.
+ * The call and everything it enqueues allocates and frees nothing.
+ *
+ *   local_counts     int32 [n_logical] or NULL, out: this GPU's tokens per logical
+ *                    expert (what the last row of lplb_plan's counts_by_block holds)
+ *
+ * Limit: n_blocks * n_logical <= 262144 counters (LPLB_EUNSUPPORTED beyond; e.g. 256
+ * slices of 1024 logical experts, 1024 slices of 256).  Every call on a GPU uses that
+ * GPU's one table, whatever the stream: calls whose kernels overlap in time on one GPU
+ * race on it.  Calls on one stream are ordered and safe.  The table keeps the previous
+ * call's contents; nothing in it needs clearing, every row is written before it is read.
+ */
+int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
+                      const int32_t *global_counts, const int32_t *r2o,
+                      const int32_t *o2r, const int32_t *phy2log, int n_group,
+                      int group_size, int dup_per_rank, int n_combined_experts,
+                      int n_local_experts, int n_blocks, int32_t *local_counts,
+                      float *global_workload, float *o_weight, int32_t *avail_num,
+                      int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
+                      lplb_stream_t stream);
 
 /*
  * No counterpart in the reference.  enabled = 0 makes lplb_plan always run the

@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1
@@ -41,6 +41,7 @@ _SIGNATURES = {
     "lplb_plan_set_cooperative": (_i, [_i]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
     "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "lplb_plan_noalloc": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
 }
 
 

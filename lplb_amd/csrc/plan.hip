@@ -592,15 +592,14 @@ extern "C" int lplb_plan_sync_timeouts(int *count) {
   return LPLB_OK;
 }
 
-extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
-                         const int32_t *global_counts, const int32_t *r2o,
-                         const int32_t *o2r, const int32_t *phy2log, int n_group,
-                         int group_size, int dup_per_rank, int n_combined_experts,
-                         int n_local_experts, int n_blocks, int32_t *counts_by_block,
-                         float *global_workload, float *o_weight, int32_t *avail_num,
-                         int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
-                         lplb_stream_t stream) {
-  using namespace lplb;
+namespace lplb {
+
+// The body of lplb_plan: argument checks, then the one-launch form or the chain.
+static int plan_checked(const int64_t *idx, int64_t n_elements, const int32_t *global_counts, const int32_t *r2o,
+                        const int32_t *o2r, const int32_t *phy2log, int n_group, int group_size, int dup_per_rank,
+                        int n_combined_experts, int n_local_experts, int n_blocks, int32_t *counts_by_block,
+                        float *global_workload, float *o_weight, int32_t *avail_num, int64_t *out,
+                        int32_t *physical_counts, int step_rule, int n_steps, lplb_stream_t stream) {
   LPLB_REQUIRE(n_group > 0 && group_size > 0 && dup_per_rank > 0 && n_blocks > 0, LPLB_EINVAL,
                "plan: n_group=%d group_size=%d dup_per_rank=%d n_blocks=%d must be positive",
                n_group, group_size, dup_per_rank, n_blocks);
@@ -650,4 +649,87 @@ extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
   return lplb_map_idx(idx, o_weight, counts_by_block, o2r, phy2log, n_elements, n_group,
                       group_size, dup_per_rank, n_combined_experts, n_local_experts, n_blocks, out,
                       physical_counts, stream);
+}
+
+// ---- the plan for callers that cannot allocate ----
+// The slice table of a plan (counts_by_block of lplb_plan: n_blocks rows of n_logical
+// counters that the workgroups exchange) lives in this array instead of a buffer of the
+// caller's.  Every GPU the library runs on holds its own copy until the process ends.
+constexpr int64_t kScratchInts = 1 << 18;   // 1 MiB: e.g. 256 slices x 1024 logical experts
+static __device__ __align__(256) int32_t scratch[kScratchInts];
+
+// Device address of `scratch` on the current device, looked up once per device (the
+// array's name is only a host-side handle; threads that race for the first look-up
+// store the same value).
+static int scratch_of_current_device(int32_t **ptr) {
+  static std::atomic<int32_t *> scratch_of[64];
+  int dev = -1;
+  LPLB_HIP_TRY(hipGetDevice(&dev));
+  LPLB_REQUIRE(dev >= 0 && dev < 64, LPLB_EUNSUPPORTED, "plan_noalloc: device ordinal %d", dev);
+  int32_t *p = scratch_of[dev].load(std::memory_order_acquire);
+  if (!p) {
+    LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    LPLB_REQUIRE(p != nullptr, LPLB_EHIP, "plan_noalloc: no device address for the slice table");
+    scratch_of[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return LPLB_OK;
+}
+
+__global__ void copy_ints(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    dst[i] = src[i];
+}
+
+} // namespace lplb
+
+extern "C" int lplb_plan(const int64_t *idx, int64_t n_elements,
+                         const int32_t *global_counts, const int32_t *r2o,
+                         const int32_t *o2r, const int32_t *phy2log, int n_group,
+                         int group_size, int dup_per_rank, int n_combined_experts,
+                         int n_local_experts, int n_blocks, int32_t *counts_by_block,
+                         float *global_workload, float *o_weight, int32_t *avail_num,
+                         int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
+                         lplb_stream_t stream) {
+  return lplb::plan_checked(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
+                            n_combined_experts, n_local_experts, n_blocks, counts_by_block, global_workload,
+                            o_weight, avail_num, out, physical_counts, step_rule, n_steps, stream);
+}
+
+extern "C" int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
+                                 const int32_t *global_counts, const int32_t *r2o,
+                                 const int32_t *o2r, const int32_t *phy2log, int n_group,
+                                 int group_size, int dup_per_rank, int n_combined_experts,
+                                 int n_local_experts, int n_blocks, int32_t *local_counts,
+                                 float *global_workload, float *o_weight, int32_t *avail_num,
+                                 int64_t *out, int32_t *physical_counts, int step_rule, int n_steps,
+                                 lplb_stream_t stream) {
+  using namespace lplb;
+  LPLB_REQUIRE(n_group > 0 && group_size > 0 && dup_per_rank > 0 && n_blocks > 0 && n_combined_experts >= 0,
+               LPLB_EINVAL, "plan_noalloc: n_group=%d group_size=%d dup_per_rank=%d n_blocks=%d must be positive",
+               n_group, group_size, dup_per_rank, n_blocks);
+  const int64_t L = (int64_t)n_local_experts - (int64_t)dup_per_rank * n_combined_experts;
+  LPLB_REQUIRE(L > 0, LPLB_EINVAL, "plan_noalloc: n_local_experts=%d does not fit %d x %d replicas", n_local_experts,
+               dup_per_rank, n_combined_experts);
+  const int64_t n_logical = (int64_t)n_group * group_size * L;
+  LPLB_REQUIRE((int64_t)n_blocks * n_logical <= kScratchInts, LPLB_EUNSUPPORTED,
+               "plan_noalloc: n_blocks=%d x %lld logical experts = %lld counters exceed the built-in slice table of "
+               "%lld; use fewer slices or lplb_plan with a workspace of your own",
+               n_blocks, (long long)n_logical, (long long)((int64_t)n_blocks * n_logical), (long long)kScratchInts);
+  int32_t *table = nullptr;
+  int rc = scratch_of_current_device(&table);
+  if (rc != LPLB_OK)
+    return rc;
+  // Nothing in the table has to start at zero: every row is written (by the slice that
+  // owns it) before anything reads it, and rows beyond n_blocks are never read.
+  rc = plan_checked(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
+                    n_combined_experts, n_local_experts, n_blocks, table, global_workload, o_weight, avail_num, out,
+                    physical_counts, step_rule, n_steps, stream);
+  if (rc != LPLB_OK || local_counts == nullptr)
+    return rc;
+  launch(copy_ints, dim3((unsigned)((n_logical + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+         table + (int64_t)(n_blocks - 1) * n_logical, local_counts, (int)n_logical);
+  LPLB_HIP_TRY(hipGetLastError());
+  return LPLB_OK;
 }
