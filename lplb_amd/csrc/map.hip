@@ -1,24 +1,28 @@
 // Logical -> physical redirect of routing indices (streaming, HBM-bound:
 // 8 bytes read + 8 bytes written per index).
 //
-// Each token needs its ordinal k among the tokens of the same expert, in index
-// order, because the original/replica decision hashes k.  The reference takes k
-// from a shared-memory atomic (minilp.cu:504), which fixes the set of ordinals
-// per block but not which token gets which.  Here k is canonical.
+// A token of an expert WITHOUT a replica goes to the expert's original slot: one
+// table look-up.  A token of an expert WITH a replica needs its ordinal k among the
+// tokens of the same expert, in index order, because the original/replica decision
+// hashes k (minilp.cu:503-509).  The reference takes k from a shared-memory atomic
+// (minilp.cu:504), which fixes the set of ordinals per block but not which token
+// gets which.  Here k is canonical, and it is worked out only for the replicated
+// sets (a few per rank), which keeps the ranking state small: one 16-byte slot per
+// (wave, replicated set, chunk).
 //
 // A workgroup walks its slice in passes of n_waves * K consecutive 64-index chunks,
-// K per wave.  The loads of the first pass are issued up front (before the small
-// table loads are used), those of every later pass while the pass before it is
-// still being ranked and stored.  Per pass:
-//   A  each wave histograms its K chunks into its own LDS counter row;
-//   B  each wave turns the rows into its starting ordinals (running total of
-//      earlier slices and passes + counts of the waves before it);
-//   C  chunk by chunk, lanes holding the same expert find each other through a
-//      per-wave 64-bit LDS bitmap (one OR, one 16-byte read); the rank among those
-//      peers is a popcount of lower lanes and the last peer advances the counter.
-// Counter rows and running totals are double-buffered by pass parity, which
-// leaves one workgroup barrier per pass.  Nothing depends on execution order.
-// The modulo of the hash uses a per-expert reciprocal prepared with the tables.
+// K per wave; the loads of two passes are in flight.  Per pass:
+//   A  every lane looks up its token's route; lanes with a replicated expert set
+//      their bit in the 64-bit bitmap of (wave, set, chunk);
+//   -- workgroup barrier --
+//   B  lane (set, chunk) counts the bits of the same set and chunk in the waves
+//      before it (popcounts) and of the chunks before it in its own wave, which gives
+//      the ordinal of the chunk's first token of that set;
+//   C  a token's ordinal is that start plus the number of lower lanes in the bitmap
+//      (one 16-byte LDS read, two mbcnt); hash, compare, store.
+// Nothing in C depends on another chunk, so the K chunks of a wave overlap.
+// Bitmaps and running totals are double-buffered by pass parity, which leaves one
+// workgroup barrier per pass.  Nothing depends on execution order.
 #include "map_kernel.h"
 
 namespace lplb {
@@ -31,7 +35,8 @@ struct MapArgs {
   const int32_t *phy2log;
   int64_t n;
   int64_t per;
-  int n_logical, n_ranks, G, D, C, L, P, n_blocks;
+  int n_logical, n_ranks, n_rep, G, D, C, L, P, n_blocks;
+  uint32_t magic_L, magic_cd, magic_D, magic_G;   // fast_div_magic of L, C * D, D, G
   int64_t *out;
   int32_t *physical_counts;   // [n_ranks * P] tokens per physical expert, or null
   long long *clocks;   // debug builds: stamps of the first and the last workgroup (else null)
@@ -45,167 +50,306 @@ __global__ void zero_ints(int32_t *p, int n) {
     p[i] = 0;
 }
 
-template <int K, bool WRAP>
+// LDS bytes for n_logical experts, n_rep replicated sets, w waves and K chunks per wave and pass.
+static size_t map_lds_bytes(int n_logical, int n_rep, int w, int k) {
+  return (size_t)(n_rep + 1) * sizeof(RepEntry) + (size_t)w * (n_rep + 1) * rank_record_bytes(k) +
+         (size_t)(n_logical + 1) * sizeof(Route) + (size_t)2 * n_rep * sizeof(int32_t) +
+         (size_t)2 * n_logical * sizeof(int32_t);
+}
+
+// TAIL: some wave's K chunks may reach past the end of its slice (loads and stores are
+// then predicated per lane); without it every pass of every slice is whole, and the
+// code from the first load to the first barrier has no branch, which lets the compiler
+// count outstanding loads exactly: the tables are built from the small loads while the
+// index loads issued after them are still in flight.
+template <int K, bool WRAP, bool TAIL>
 __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  const int nl = a.n_logical;
+  constexpr int kRec = rank_record_bytes(K);
+  const int nl = a.n_logical, R = a.n_rep;
   const int tid = threadIdx.x, nt = blockDim.x;
-  const int lane = tid % kWave, wave = tid / kWave, n_waves = nt / kWave;
-  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, but known to be wave-uniform
+  const int lane = tid % kWave, n_waves = nt / kWave;
+  const int wave_s = __builtin_amdgcn_readfirstlane(tid / kWave);   // wave-uniform
   const int pid = blockIdx.x;
-  ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);                 // [nl]
-  WaveSlot *slots = reinterpret_cast<WaveSlot *>(table + nl);                    // [n_waves][nl]
-  int32_t *replica = reinterpret_cast<int32_t *>(slots + (size_t)n_waves * nl);  // [nl]
-  int32_t *carry = replica + nl;                                                 // [2][nl]
-  int32_t *counts = carry + 2 * nl;                                              // [2][n_waves][nl]
-  const int32_t *last = a.by_block + (int64_t)(a.n_blocks - 1) * nl;
-  const int32_t *prev = pid ? a.by_block + (int64_t)(pid - 1) * nl : nullptr;
-
   const int64_t begin = slice_begin(a.n, a.per, pid);
   const int64_t end = slice_begin(a.n, a.per, pid + 1);
-  const int64_t pass_len = (int64_t)n_waves * K * kWave;
-  WaveSlot *mine = slots + (size_t)wave * nl;
+  const bool counts_wanted = pid == 0 && a.physical_counts != nullptr;
+  if (begin >= end && !counts_wanted)
+    return;
+
+  RepEntry *reps = reinterpret_cast<RepEntry *>(smem_raw);                          // [R + 1]
+  unsigned char *records = smem_raw + (size_t)(R + 1) * sizeof(RepEntry);          // [n_waves][R + 1][kRec]
+  const int wave_stride = (R + 1) * kRec;
+  Route *route = reinterpret_cast<Route *>(records + (size_t)n_waves * wave_stride);   // [nl + 1]
+  int32_t *carry = reinterpret_cast<int32_t *>(route + nl + 1);                     // [2][R]
+  int32_t *staged = carry + 2 * R;   // [2][nl] tokens per expert: in the whole array, before this slice
+  unsigned char *my_records = records + (size_t)wave_s * wave_stride;
   const unsigned long long my_bit = 1ull << lane;
+  const int32_t *last = a.by_block + (int64_t)(a.n_blocks - 1) * nl;
+  const int32_t *prev = pid ? a.by_block + (int64_t)(pid - 1) * nl : nullptr;
+  const int cd = a.C * a.D;
   LPLB_MAP_STAMP(0);
 
-  // Global reads of the table build (small, mostly L2 hits) go out first, the
-  // first pass's indices right behind them, so that the build does not wait for
-  // the bulk data.  Tables, minilp.cu:466-496.
-  const int cd = a.C * a.D;
-  const int e0 = tid;                                   // first (usually only) expert of this thread
-  const int32_t t0 = e0 < nl ? last[e0] : 0;
-  const int32_t s0 = (e0 < nl && prev) ? prev[e0] : 0;
-  const int le0 = e0 < nl ? a.phy2log[(e0 / a.L) * a.P + (e0 % a.L)] : -1;
-  const bool rep0 = tid < a.n_ranks * cd;               // first replicated expert set of this thread
-  const int rank0 = rep0 ? tid / cd : 0, local0 = rep0 ? tid % cd : 0;
-  const int rle0 = rep0 ? a.phy2log[rank0 * a.P + local0] : -1;
-  const float share0 = rep0 ? a.o_weight[rank0 * a.D + local0 % a.D] : 0.0f;
-  const int host0 = rep0 ? a.o2r[(rank0 % a.G) * a.D + local0 % a.D] : 0;
+  // ---- small global reads of the table build first (mostly L2 hits), minilp.cu:466-496 ----
+  // original slot of logical position e: rank e / L, place e % L
+  auto slot_of = [&](int e) { return e + (int)fast_div((uint32_t)e, a.magic_L) * (a.P - a.L); };
+  // replicated set i = (ep_rank, place): its expert, its share, the group rank that holds the copy
+  struct SetOf {
+    int ep_rank, place, d, group_rank;
+  };
+  auto set_of = [&](int i) {
+    SetOf s;
+    s.ep_rank = (int)fast_div((uint32_t)i, a.magic_cd);
+    s.place = i - s.ep_rank * cd;
+    s.d = s.place - (int)fast_div((uint32_t)s.place, a.magic_D) * a.D;
+    s.group_rank = s.ep_rank - (int)fast_div((uint32_t)s.ep_rank, a.magic_G) * a.G;
+    return s;
+  };
+  // All of them are unconditional loads from clamped addresses: a load inside a branch
+  // makes the compiler wait for it right there, before the index loads are issued.
+  const int e0 = min(tid, nl - 1);                          // first (usually only) expert of this thread
+  const int slot0 = slot_of(e0);
+  const int le0 = a.phy2log[slot0];
+  // The counts are read per expert, not per replicated set, so that they do not have to
+  // wait for phy2log (a load issued after the index loads returns after them).
+  const int32_t total0 = last[e0];
+  const int32_t before0_raw = (prev ? prev : last)[e0];
+  const bool set0 = tid < R;                               // first (usually only) replicated set
+  const SetOf s0 = set_of(set0 ? tid : 0);
+  // (with no replicated set at all, R == 0, these read element 0 of each table)
+  const int rle0 = a.phy2log[s0.ep_rank * a.P + s0.place];
+  const float share0 = a.o_weight[s0.ep_rank * a.D + s0.d];
+  const int host0 = a.o2r[s0.group_rank * a.D + s0.d];
 
-  // One pass of indices, as loaded (raw) and as expert ids (ev: -1 for masked /
-  // out-of-range / past the end).  The loads of the next pass are issued while the
-  // current one is still being ranked and stored.
-  int64_t raw[K];
-  int32_t ev[K];
-  auto issue_loads = [&](int64_t pass) {
+  // ---- the index loads of the first two passes right behind them ----
+  const int64_t pass_len = (int64_t)n_waves * K * kWave;
+  const int64_t wave_off = (int64_t)wave_s * (K * kWave);
+  auto issue_loads = [&](int64_t (&raw)[K], int64_t pass) {
+    const int64_t w0 = pass + wave_off;                    // first index of this wave's K chunks (uniform)
+    const int64_t *src = a.idx + w0 + lane;
+    if (!TAIL || w0 + K * kWave <= end) {
 #pragma unroll
-    for (int c = 0; c < K; ++c) {
-      const int64_t i = pass + ((int64_t)wave * K + c) * kWave + lane;
-      raw[c] = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
+      for (int c = 0; c < K; ++c)
+        raw[c] = __builtin_nontemporal_load(src + c * kWave);
+    } else {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        raw[c] = w0 + c * kWave + lane < end ? __builtin_nontemporal_load(src + c * kWave) : -1;
     }
   };
-  auto take_loads = [&]() {
-#pragma unroll
-    for (int c = 0; c < K; ++c)
-      ev[c] = (raw[c] >= 0 && raw[c] < nl) ? (int32_t)raw[c] : -1;
-  };
-  issue_loads(begin);
+  int64_t raw0[K], raw1[K];
+  issue_loads(raw0, begin);
+  // (without TAIL a slice of one pass loads that pass twice rather than branch here)
+  issue_loads(raw1, (TAIL || begin + pass_len < end) ? begin + pass_len : begin);
 
-  const RedirectShape sh{nl, a.n_ranks, a.G, a.D, a.C, a.L, a.P};
-  if (e0 < nl)
-    init_entry(table, replica, carry, e0, t0, s0);
-  for (int e = tid + nt; e < nl; e += nt)
-    init_entry(table, replica, carry, e, last[e], prev ? prev[e] : 0);
-  for (int i = tid; i < n_waves * nl; i += nt) {
-    slots[i] = WaveSlot{0, 0, 0ull};
-    counts[i] = 0;
-    counts[n_waves * nl + i] = 0;
+  // ---- tables ----
+  for (int e = tid; e <= nl; e += nt)
+    route[e] = Route{-1, R};
+  {
+    const i32x4 zero{0, 0, 0, 0};
+    i32x4 *z = reinterpret_cast<i32x4 *>(records);
+    for (int i = tid; i < n_waves * wave_stride / 16; i += nt)
+      z[i] = zero;
+  }
+  if (tid == 0)
+    reps[R] = RepEntry{1, 0xffffffffu, INT32_MAX, -1};   // "no replica": every token stays
+  if (tid < nl) {
+    staged[tid] = total0;
+    staged[nl + tid] = prev ? before0_raw : 0;
+  }
+  for (int e = tid + nt; e < nl; e += nt) {
+    staged[e] = last[e];
+    staged[nl + e] = prev ? prev[e] : 0;
   }
   __syncthreads();
-  if (e0 < nl)
-    set_original(table, sh, e0, le0);
-  for (int e = tid + nt; e < nl; e += nt)
-    set_original(table, sh, e, a.phy2log[(e / a.L) * a.P + (e % a.L)]);
-  if (rep0)
-    set_replica(table, replica, sh, rank0, local0, rle0, share0, host0);
-  for (int i = tid + nt; i < a.n_ranks * cd; i += nt) {
-    const int ep_rank = i / cd, local = i % cd, d = local % a.D;
-    set_replica(table, replica, sh, ep_rank, local, a.phy2log[ep_rank * a.P + local],
-                a.o_weight[ep_rank * a.D + d], a.o2r[(ep_rank % a.G) * a.D + d]);
+  if (tid < nl && le0 >= 0 && le0 < nl)
+    route[le0].original = slot0;
+  for (int e = tid + nt; e < nl; e += nt) {
+    const int s = slot_of(e), le = a.phy2log[s];
+    if (le >= 0 && le < nl)
+      route[le].original = s;
   }
-  // (the barrier after the first phase A also publishes the tables)
+  // A set's key is R - 1 - i, so that of two sets that name the same expert the later one
+  // wins (as a sequential pass over the sets would have it) with an atomic min.
+  auto fill_set = [&](int i, const SetOf &s, int le, float share, int host) {
+    const bool ok = le >= 0 && le < nl;
+    const int32_t t = ok ? staged[le] : 0;
+    const int32_t before = ok ? staged[nl + le] : 0;
+    if (ok)
+      atomicMin(&route[le].rep, R - 1 - i);
+    RepEntry x;
+    x.total = t;
+    x.magic = t >= 1 ? 0xffffffffu / (uint32_t)t : 0u;
+    x.expected = expected_on_original(share, t);
+    x.replica = ((s.ep_rank - s.group_rank) + host + 1) * a.P - cd + s.place;
+    reps[R - 1 - i] = x;
+    carry[R - 1 - i] = before;
+  };
+  if (set0)
+    fill_set(tid, s0, rle0, share0, host0);
+  for (int i = tid + nt; i < R; i += nt) {
+    const SetOf s = set_of(i);
+    fill_set(i, s, a.phy2log[s.ep_rank * a.P + s.place], a.o_weight[s.ep_rank * a.D + s.d],
+             a.o2r[s.group_rank * a.D + s.d]);
+  }
+  __syncthreads();
   LPLB_MAP_STAMP(1);
-
-  int parity = 0;   // which half of counts / carry the current pass uses
-  for (int64_t pass = begin; pass < end; pass += pass_len) {
-    take_loads();
-    int32_t *my_counts = counts + ((size_t)parity * n_waves + wave) * nl;
-    // Phase A: tokens per expert in this wave's chunks.
-#pragma unroll
-    for (int c = 0; c < K; ++c)
-      if (ev[c] >= 0)
-        atomicAdd(&my_counts[ev[c]], 1);
-    if (pass + pass_len < end)
-      issue_loads(pass + pass_len);   // in flight during the barrier, phases B and C
-    LPLB_MAP_STAMP(2);
-    __syncthreads();
-    LPLB_MAP_STAMP(3);
-    // Phase B: every wave derives its own starting ordinals: the running total
-    // of earlier slices and passes plus the counts of the waves before it.  The
-    // last wave writes the next pass's running total into the other half, and
-    // every wave clears its row of the other half for the next pass.
-    const int32_t *pass_counts = counts + (size_t)parity * n_waves * nl;
-    int32_t *other_counts = counts + ((size_t)(parity ^ 1) * n_waves + wave) * nl;
-    // The code is specialised by the number of earlier waves (wave-uniform), so that
-    // the inner loop is straight-line: exactly that many reads, no branches.
-    static_for<kMaxWaves>([&](auto wc) {
-      constexpr int kEarlier = decltype(wc)::value;
-      if (wave_s != kEarlier)
-        return;
-      for (int e = lane; e < nl; e += kWave) {
-        // all reads in flight before the first add
-        int32_t before[kEarlier + 1];
-#pragma unroll
-        for (int w = 0; w < kEarlier; ++w)
-          before[w] = pass_counts[(size_t)w * nl + e];
-        int32_t run = carry[parity * nl + e];
-        const int32_t own = my_counts[e];
-#pragma unroll
-        for (int w = 0; w < kEarlier; ++w)
-          run += before[w];
-        mine[e].next = run;
-        if (kEarlier == n_waves - 1)
-          carry[(parity ^ 1) * nl + e] = run + own;
-        other_counts[e] = 0;
+  // Tokens per physical expert (= bincount of the output) from the tables alone.
+  if (counts_wanted)
+    for (int i = tid; i < a.n_ranks * a.P; i += nt) {
+      const int le = a.phy2log[i];
+      int32_t v = 0;
+      if (le >= 0 && le < nl) {
+        const Route rt = route[le];
+        if (rt.rep >= R) {
+          v = rt.original == i ? staged[le] : 0;
+        } else {
+          const RepEntry x = reps[rt.rep];
+          const int32_t kept = kept_on_original(x.total, x.expected);
+          v = rt.original == i ? kept : (x.replica == i ? x.total - kept : 0);
+        }
       }
-    });
-    __builtin_amdgcn_wave_barrier();
-    LPLB_MAP_STAMP(4);
-    // Phase C.
+      a.physical_counts[i] = v;
+    }
+
+  // ---- one pass ----
+  auto process = [&](auto parity_c, int64_t (&raw)[K], int64_t pass) {
+    constexpr int PAR = decltype(parity_c)::value;
+    int32_t original[K];
+    int32_t set[K];
 #pragma unroll
     for (int c = 0; c < K; ++c) {
-      const int64_t o = redirect_token<WRAP>(ev[c], mine, table, replica, my_bit);
-      const int64_t i = pass + ((int64_t)wave * K + c) * kWave + lane;
-      if (i < end)
-        __builtin_nontemporal_store(o, a.out + i);
-      __builtin_amdgcn_wave_barrier();
+      const bool valid = (uint64_t)raw[c] < (uint64_t)nl;   // -1, other negatives and too large ids fail
+      const Route rt = route[valid ? (int)raw[c] : nl];
+      original[c] = rt.original;
+      set[c] = rt.rep;
     }
-    LPLB_MAP_STAMP(5);
-    parity ^= 1;
+    if (pass + 2 * pass_len < end)
+      issue_loads(raw, pass + 2 * pass_len);   // in flight during this pass and the next
+    // Phase A.
+    ChunkSlot *slot[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      slot[c] = reinterpret_cast<ChunkSlot *>(my_records + __umul24((uint32_t)set[c], (uint32_t)kRec)) + (PAR * K + c);
+      if (set[c] < R)
+        atomicOr(reinterpret_cast<unsigned long long *>(slot[c]), my_bit);
+    }
+    LPLB_MAP_STAMP(2 + 4 * PAR);
+    __syncthreads();
+    LPLB_MAP_STAMP(3 + 4 * PAR);
+    // Phase B: lane = (set, chunk), chunk fastest.  The rows of the waves before this
+    // one are read four at a time (clamped addresses, masked values).
+    if (R > 0) {
+      const int c = lane % K;
+      for (int p0 = 0; p0 < R * K; p0 += kWave) {
+        const bool live = p0 + lane < R * K;
+        const int q = live ? (p0 + lane) / K : R;   // lanes past the end read the stand-in record (zeros)
+        unsigned char *first = records + __umul24((uint32_t)q, (uint32_t)kRec) + (PAR * K + c) * (int)sizeof(ChunkSlot);
+        const int32_t carried = carry[PAR * R + (live ? q : 0)];
+        const unsigned long long own_bits =
+            *reinterpret_cast<const unsigned long long *>(first + wave_s * wave_stride);
+        int earlier = 0;
+        for (int w0 = 0; w0 < wave_s; w0 += 4) {
+          unsigned long long bits[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            bits[u] = *reinterpret_cast<const unsigned long long *>(first + min(w0 + u, wave_s) * wave_stride);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            earlier += w0 + u < wave_s ? __popcll(bits[u]) : 0;
+        }
+        const int own = __popcll(own_bits);
+        const int in_earlier_waves = group_sum<K>(earlier);
+        const int in_my_wave = group_sum<K>(own);
+        const int in_earlier_chunks = group_exclusive_scan<K>(own, c);
+        if (live) {
+          const int32_t base = carried + in_earlier_waves;
+          ChunkSlot *mine = reinterpret_cast<ChunkSlot *>(first + wave_s * wave_stride);
+          mine->start = base + in_earlier_chunks;
+          // the other parity's bitmap is free again: clear it for the pass after this one
+          *reinterpret_cast<unsigned long long *>(mine + (PAR ? -K : K)) = 0ull;
+          if (wave_s == n_waves - 1 && c == 0)
+            carry[(PAR ^ 1) * R + q] = base + in_my_wave;
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    LPLB_MAP_STAMP(4 + 4 * PAR);
+    // Phase C: all LDS reads of the K chunks first, then the arithmetic, then the stores.
+    const int64_t w0 = pass + wave_off;
+    int64_t *dst = a.out + w0 + lane;
+    i32x4 s[K], x[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      s[c] = *reinterpret_cast<const i32x4 *>(slot[c]);         // bits_lo, bits_hi, start
+      x[c] = *reinterpret_cast<const i32x4 *>(&reps[set[c]]);   // total, magic, expected, replica
+    }
+    int32_t o[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const int32_t k = __builtin_amdgcn_mbcnt_hi((uint32_t)s[c].y,
+                                                  __builtin_amdgcn_mbcnt_lo((uint32_t)s[c].x, (uint32_t)s[c].z));
+      const int32_t h = ordinal_hash<WRAP>(k, x[c].x, (uint32_t)x[c].y);
+      o[c] = h >= x[c].z ? x[c].w : original[c];
+    }
+    if (!TAIL || w0 + K * kWave <= end) {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        __builtin_nontemporal_store((int64_t)o[c], dst + c * kWave);
+    } else {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        if (w0 + c * kWave + lane < end)
+          __builtin_nontemporal_store((int64_t)o[c], dst + c * kWave);
+    }
+    LPLB_MAP_STAMP(5 + 4 * PAR);
+  };
+
+  for (int64_t pass = begin; pass < end; pass += 2 * pass_len) {
+    process(std::integral_constant<int, 0>{}, raw0, pass);
+    if (pass + pass_len >= end)
+      break;
+    process(std::integral_constant<int, 1>{}, raw1, pass + pass_len);
   }
-  if (pid == 0 && a.physical_counts)   // the tables are complete since the first barrier
-    emit_physical_counts(table, replica, sh, a.phy2log, a.physical_counts, tid, nt);
+
+#ifdef LPLB_PHASE_CLOCKS
   __builtin_amdgcn_s_waitcnt(0);
-  LPLB_MAP_STAMP(6);
+#endif
+  LPLB_MAP_STAMP(10);
 }
 
-// LDS bytes for n_logical experts and w waves.
-static size_t map_lds_bytes(int n_logical, int w) {
-  return (size_t)n_logical * (sizeof(ExpertEntry) + 4 + 8 + (size_t)w * (sizeof(WaveSlot) + 8));
-}
+#ifdef LPLB_TUNING
+// Tuning builds only: force the launch shape of the redirect (0 = choose as usual).
+int g_force_waves = 0, g_force_k = 0;
+#endif
 
-template <int K, bool WRAP>
-static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+template <int K, bool WRAP, bool TAIL>
+static hipError_t launch_redirect_variant(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
   if (lds > 64 * 1024) {
-    const hipError_t err = allow_dynamic_lds(&redirect_indices<K, WRAP>, 160 * 1024);
+    const hipError_t err = allow_dynamic_lds(&redirect_indices<K, WRAP, TAIL>, 160 * 1024);
     if (err != hipSuccess)
       return err;
   }
-  launch(redirect_indices<K, WRAP>, grid, block, lds, s, a);
+  launch(redirect_indices<K, WRAP, TAIL>, grid, block, lds, s, a);
   return hipGetLastError();
+}
+template <int K, bool WRAP>
+static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
+  // every slice a whole number of passes?  (the last slice may be shorter than the others)
+  const int64_t pass_len = (int64_t)block.x * K;
+  const bool whole = a.per % pass_len == 0 && a.n % pass_len == 0;
+  return whole ? launch_redirect_variant<K, WRAP, false>(a, grid, block, lds, s)
+               : launch_redirect_variant<K, WRAP, true>(a, grid, block, lds, s);
 }
 
 } // namespace lplb
+
+#ifdef LPLB_TUNING
+extern "C" void lplb_debug_force_redirect_shape(int waves, int k) {
+  lplb::g_force_waves = waves;
+  lplb::g_force_k = k;
+}
+#endif
 
 extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
                             const int32_t *counts_by_block, const int32_t *o2r,
@@ -245,49 +389,60 @@ extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
   a.idx = idx; a.o_weight = o_weight; a.by_block = counts_by_block; a.o2r = o2r;
   a.phy2log = phy2log; a.n = n_elements; a.per = slice_len(n_elements, n_blocks);
   a.n_ranks = n_group * group_size; a.n_logical = a.n_ranks * L;
+  a.n_rep = a.n_ranks * n_combined_experts * dup_per_rank;
   a.G = group_size; a.D = dup_per_rank; a.C = n_combined_experts; a.L = L;
   a.P = n_local_experts; a.n_blocks = n_blocks; a.out = out; a.physical_counts = physical_counts;
+  LPLB_REQUIRE(a.n_logical < 65536 && a.n_ranks * a.P < 65536, LPLB_EUNSUPPORTED,
+               "map_idx: %d logical / %d physical experts exceed the 65535 the tables index", a.n_logical,
+               a.n_ranks * a.P);
+  a.magic_L = fast_div_magic((uint32_t)L);
+  a.magic_cd = fast_div_magic((uint32_t)(n_combined_experts * dup_per_rank));
+  a.magic_D = fast_div_magic((uint32_t)dup_per_rank);
+  a.magic_G = fast_div_magic((uint32_t)group_size);
 #ifdef LPLB_PHASE_CLOCKS
   a.clocks = g_phase_clocks;
 #else
   a.clocks = nullptr;
 #endif
 
-  // One wave per 64-index chunk of the slice, as LDS allows, then up to 8 chunks per
-  // wave and pass.  At most 16 waves when there is one workgroup per CU; with more
-  // workgroups than CUs smaller ones (8, then 4 waves) share a CU, and one's ranking
-  // phases overlap another's loads and stores (measured at 512 MiB in + 512 MiB out:
-  // 1024 slices of 4 waves 4.9 TB/s, 256 slices of 16 waves 4.1 TB/s).
+  // Waves per workgroup: one per 64-index chunk of the slice, at most 16 when there is
+  // one workgroup per CU; with more workgroups than CUs smaller ones (8, then 4 waves)
+  // share a CU.  A wave takes K chunks per pass; two passes are in flight, so that one
+  // pass's ranking and stores overlap the next one's loads.
   const int64_t chunks = (a.per + kWave - 1) / kWave;
   const int n_cus = current_device_cu_count();
   int max_waves = kMaxWaves;
   while (max_waves > 4 && n_cus > 0 && (int64_t)n_blocks * max_waves > (int64_t)kMaxWaves * n_cus)
     max_waves >>= 1;
   int n_waves = chunks < max_waves ? (int)chunks : max_waves;
-  constexpr size_t kLdsLimit = 160 * 1024;
-  while (n_waves > 1 && map_lds_bytes(a.n_logical, n_waves) > kLdsLimit)
-    n_waves >>= 1;
-  LPLB_REQUIRE(map_lds_bytes(a.n_logical, n_waves) <= kLdsLimit, LPLB_EUNSUPPORTED,
-               "map_idx: %d logical experts do not fit the LDS tables", a.n_logical);
   const int64_t per_wave = (chunks + n_waves - 1) / n_waves;
-  const size_t lds = map_lds_bytes(a.n_logical, n_waves);
+  int k = per_wave >= 8 ? 4 : per_wave >= 3 ? 2 : 1;
+#ifdef LPLB_TUNING
+  if (g_force_waves > 0)
+    n_waves = min(g_force_waves, kMaxWaves);
+  if (g_force_k > 0)
+    k = g_force_k;
+#endif
+  constexpr size_t kLdsLimit = 160 * 1024;
+  while (k > 1 && map_lds_bytes(a.n_logical, a.n_rep, n_waves, k) > kLdsLimit)
+    k >>= 1;
+  while (n_waves > 1 && map_lds_bytes(a.n_logical, a.n_rep, n_waves, k) > kLdsLimit)
+    n_waves >>= 1;
+  const size_t lds = map_lds_bytes(a.n_logical, a.n_rep, n_waves, k);
+  LPLB_REQUIRE(lds <= kLdsLimit, LPLB_EUNSUPPORTED,
+               "map_idx: %d logical experts with %d replicated sets do not fit the LDS tables", a.n_logical,
+               a.n_rep);
   const dim3 grid(n_blocks), block(n_waves * kWave);
   hipError_t err;
 #define LPLB_MAP_CASE(K)                                                                    \
   err = wrap ? launch_redirect<K, true>(a, grid, block, lds, s)                             \
              : launch_redirect<K, false>(a, grid, block, lds, s)
-  // K chunks per wave and pass (K loads in flight per lane, K more prefetched).
-  // Measured at [262144 x 8] on MI355X: a pass costs about 2.5 us of barrier skew
-  // and counter traffic, so a pass is as long as registers allow (8 chunks per
-  // wave); longer slices loop over passes.
-  if (per_wave <= 1) {
+  if (k <= 1) {
     LPLB_MAP_CASE(1);
-  } else if (per_wave <= 2) {
+  } else if (k <= 2) {
     LPLB_MAP_CASE(2);
-  } else if (per_wave <= 4) {
-    LPLB_MAP_CASE(4);
   } else {
-    LPLB_MAP_CASE(8);
+    LPLB_MAP_CASE(4);
   }
 #undef LPLB_MAP_CASE
   LPLB_HIP_TRY(err);

@@ -157,4 +157,88 @@ __device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntr
   return o;
 }
 
+// ---------------------------------------------------------------------------
+// Redirect with ordinals only where they matter.
+//
+// The ordinal k of a token decides between original and replica, so only tokens of
+// experts that HAVE a replica need one: every other expert's tokens go to its
+// original slot whatever k is (expected == total, minilp.cu:466-470).  The tables
+// are therefore split: a route per logical expert (original slot + index of its
+// replicated set, if any) and, per replicated set, the constants of the hash test.
+// Ranking state exists per replicated set only, which is what keeps it small.
+
+// Per logical expert; entry n_logical is the route of masked / out-of-range tokens.
+struct __attribute__((aligned(8))) Route {
+  int32_t original;  // physical slot of the original, -1 if none
+  int32_t rep;       // index of the replicated set this expert belongs to; n_rep if it has no replica
+};
+// Per replicated set (ep_rank, slot) in the order of minilp.cu:478-495; entry n_rep is a
+// stand-in for "no replica" whose test never sends a token away (expected = INT32_MAX).
+struct __attribute__((aligned(16))) RepEntry {
+  int32_t total;     // tokens of the expert in the whole index array
+  uint32_t magic;    // floor((2^32 - 1) / total), 0 for total <= 0
+  int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
+  int32_t replica;   // physical slot of the replica
+};
+// One 64-index chunk of one wave and one replicated set.
+struct __attribute__((aligned(16))) ChunkSlot {
+  uint32_t bits_lo, bits_hi;  // lanes of the chunk that hold a token of the set
+  int32_t start;              // ordinal of the first of them
+  int32_t unused;
+};
+
+// Bytes of the ranking record of one (wave, replicated set): K chunk slots for each of
+// the two pass parities, padded to an odd multiple of 16 bytes so that consecutive
+// sets start in different LDS banks.
+constexpr int rank_record_bytes(int k) { return 2 * k * (int)sizeof(ChunkSlot) + 16; }
+
+// (499 k + 41) mod total with the sign rule of C (minilp.cu:505), k >= 0.
+// !WRAP: k < 2^24 and 499 k + 41 < 2^31 (the caller guarantees it).
+template <bool WRAP> __device__ inline int32_t ordinal_hash(int32_t k, int32_t total, uint32_t magic) {
+  if constexpr (WRAP) {
+    ExpertEntry x;
+    x.total = total;
+    x.magic = magic;
+    return hashed_mod<true>((int32_t)((uint32_t)k * 499u + 41u), x);
+  } else {
+    const uint32_t a = __umul24((uint32_t)k, 499u) + 41u;
+    const uint32_t r = a - __umulhi(a, magic) * (uint32_t)total;   // true remainder, or that plus total
+    return (int32_t)min(r, r - (uint32_t)total);
+  }
+}
+
+// Exact n / d for n < 65536 and 1 <= d < 65536 with m = fast_div_magic(d) =
+// floor(2^32 / d) + 1: m d = 2^32 + delta with 0 < delta <= d, so n m / 2^32 exceeds
+// n / d by n delta / (d 2^32) < 1 / d, too little to reach the next integer.  d = 1
+// (m would be 2^32 + 1) is encoded as m = 0.
+__host__ __device__ inline uint32_t fast_div_magic(uint32_t d) {
+  return d <= 1 ? 0u : (uint32_t)(0x100000000ull / d) + 1u;
+}
+__device__ inline uint32_t fast_div(uint32_t n, uint32_t m) { return m ? __umulhi(n, m) : n; }
+
+// DPP row shift right by N lanes inside a row of 16 (lanes without a source get 0).
+template <int N> __device__ inline int row_shr(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, 0x110 + N, 0xF, 0xF, true);
+}
+template <int CTRL> __device__ inline int dpp_int(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+// Sum over each group of K adjacent lanes (K = 1, 2, 4 or 8; every lane gets its group's sum).
+template <int K> __device__ inline int group_sum(int v) {
+  if constexpr (K >= 2) v += dpp_int<0xB1>(v);    // quad_perm [1,0,3,2]
+  if constexpr (K >= 4) v += dpp_int<0x4E>(v);    // quad_perm [2,3,0,1]
+  if constexpr (K >= 8) v += dpp_int<0x141>(v);   // row_half_mirror
+  return v;
+}
+// Sum of the lanes before this one in its group of K adjacent lanes (pos = lane % K).
+template <int K> __device__ inline int group_exclusive_scan(int v, int pos) {
+  int acc = 0;
+  static_for<K - 1>([&](auto jc) {
+    constexpr int j = decltype(jc)::value + 1;
+    const int from_left = row_shr<j>(v);
+    acc += pos >= j ? from_left : 0;
+  });
+  return acc;
+}
+
 } // namespace lplb
