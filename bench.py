@@ -31,11 +31,24 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 REDIRECT_BYTES_PER_INDEX = 16
-# HBM bytes one redirect launch moves at the sweep shape, from rocprofv3 FETCH_SIZE and WRITE_SIZE (two
-# runs), each scaled by what the same counter reads for the plain copy kernel of known size:
-# 16 797 KiB read + 16 376 KiB written, 1.012 x the algorithmic bytes.
-REDIRECT_TRAFFIC_BYTES_SWEEP = 34_341_000
 HISTOGRAM_BYTES_PER_INDEX = 8
+# HBM bytes one redirect launch moves at the sweep shape come from rocprofv3 counters (FETCH_SIZE and
+# WRITE_SIZE, two runs, each scaled by what the same counter reads for the plain copy kernel of known
+# size).  They cannot be measured from inside this script, so the figure is read from the tracked
+# summary of that measurement, which also names the commit whose kernel it was taken from.
+TRAFFIC_SUMMARY = ROOT / "profiles" / "redirect_sweep_262144x8_hbm_traffic.md"
+
+
+def measured_redirect_traffic():
+    """(bytes per launch, commit the kernel was measured at) from the profile summary, or (None, None)."""
+    import re
+    try:
+        text = TRAFFIC_SUMMARY.read_text()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
+    c = re.search(r"measured_at_commit:\s*([0-9a-f]+)", text)
+    return (int(m.group(1)) if m else None), (c.group(1) if c else None)
 
 
 def pct(a, q):
@@ -250,8 +263,10 @@ def main() -> None:
             assert lib.lplb_copy_calibration(bufs_in[i].data_ptr(), bufs_out[i].data_ptr(), n_idx, stream) == 0
     copy_us = timer.times_us(torch)
     copy_gbs = alg_bytes / (float(copy_us.mean()) * 1e-6) / 1e9
+    traffic, traffic_commit = measured_redirect_traffic()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": REDIRECT_TRAFFIC_BYTES_SWEEP,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_measured_at_commit": traffic_commit,
                 "kernel": "redirect_indices",
                 "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64, {roof_blocks} slices",
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
@@ -286,6 +301,38 @@ def main() -> None:
         h_us = event_times_us(hist_next, 10 * n_buf, n_buf, torch)
         extras["histogram_sweep_us"] = round(float(h_us.mean()), 2)
         extras["histogram_sweep_GBs"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (float(h_us.mean()) * 1e-6) / 1e9, 1)
+        extras["histogram_sweep_frac_of_peak"] = round(extras["histogram_sweep_GBs"] / HBM_PEAK_GBS, 4)
+        # the histogram kernel alone (without the scan over slices that follows it), by its own timestamps
+        h_timer = KernelTimer(lib, 4 * n_buf)
+        for r in range(4 * n_buf):
+            h_timer.arm()          # the first kernel of the call is the histogram
+            hist(r % n_buf)
+        hk_us = float(h_timer.times_us(torch).mean())
+        h_timer.close()
+        extras["histogram_kernel_sweep_us"] = round(hk_us, 2)
+        extras["histogram_kernel_sweep_frac_of_peak"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (hk_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+
+        # the whole plan at the sweep shape: histogram of [262144 x 8], LP, redirect (16 B per index)
+        sweep_counts_dev = to_dev(sweep.global_counts)
+        sw_gw = torch.empty(cfg.n_logical, dtype=torch.float32, device=dev)
+        sw_ow = torch.empty(1, G, D, dtype=torch.float32, device=dev)
+
+        def plan_sweep(i, counts_ptr):
+            rc = lib.lplb_plan(bufs_in[i].data_ptr(), n_idx, counts_ptr, r2o.data_ptr(), o2r.data_ptr(),
+                               sweep_p2l.data_ptr(), 1, G, D, C, P, roof_blocks, tables[i].data_ptr(), sw_gw.data_ptr(),
+                               sw_ow.data_ptr(), avail.data_ptr(), bufs_out[i].data_ptr(), None, 0, 5, stream)
+            assert rc == 0, lib.lplb_last_error()
+        for tag, ptr in (("", sweep_counts_dev.data_ptr()), ("_own_histogram", None)):
+            turn_s = [0]
+
+            def plan_sweep_next():
+                plan_sweep(turn_s[0] % n_buf, ptr)
+                turn_s[0] += 1
+            ps_us = event_times_us(plan_sweep_next, 10 * n_buf, n_buf, torch)
+            extras[f"plan_sweep_shape{tag}_us_p50"] = round(pct(ps_us, 50), 2)
+            extras[f"plan_sweep_shape{tag}_us_p99"] = round(pct(ps_us, 99), 2)
+        extras["plan_sweep_shape_frac_of_peak"] = round(
+            n_idx * REDIRECT_BYTES_PER_INDEX / (extras["plan_sweep_shape_us_p50"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
 
         # redirect on a batch 16x the sweep (512 MiB in, 512 MiB out): the fixed cost per launch fades
         big_n, big_slices = 16 * n_idx, 4 * n_sms
@@ -402,6 +449,54 @@ def main() -> None:
         b_us = event_times_us(batched, 100, 10, torch)
         extras["batched_2048_solves_us"] = round(pct(b_us, 50), 2)
         extras["batched_plans_per_s"] = round(2048 / (pct(b_us, 50) * 1e-6), 1)
+        # the timed launches' results, all 2048 of them, against the CPU checker (outside any timed region)
+        avail.zero_()
+        batched()
+        torch.cuda.synchronize()
+        b_flow, b_obj, b_ok = oracle.compare_batch(synth.sweep_counts(2048), results.cpu().numpy(), cfg.r2o, inp.phy2log,
+                                                   1, C, n_fixed)
+        assert b_flow <= 1e-4 and b_obj <= 1e-3 and int(avail[0]) == b_ok == 2048, (b_flow, b_obj, b_ok, int(avail[0]))
+        extras["batched_2048_worst_flow_diff_vs_checker"] = float(f"{b_flow:.2e}")
+        extras["batched_2048_worst_objective_diff_vs_checker"] = float(f"{b_obj:.2e}")
+
+        # every other configuration of the benchmark suite: p50 / p99 per plan (global counts supplied, as
+        # one launch and as the chain of kernels) and the LP kernel's own duration
+        per_cfg = {}
+        for name in ("cpu_ref_ep8", "v3_ep8_cube", "ep16_hypercube", "ep32_torus"):
+            ci = synth.make_inputs(name)
+            cc = ci.cfg
+            g2, d2 = cc.r2o.shape
+            l2, p2 = cc.n_logical // cc.ep_size, cc.n_physical // cc.ep_size
+            c2 = (p2 - l2) // d2
+            ng = cc.ep_size // g2
+            t_r2o, t_o2r = to_dev(cc.r2o), to_dev(np.argsort(cc.r2o, axis=0, kind="stable").astype(np.int32))
+            t_p2l, t_idx, t_cnt = to_dev(ci.phy2log), to_dev(ci.indices), to_dev(ci.global_counts)
+            t_by = torch.empty(n_sms, cc.n_logical, dtype=torch.int32, device=dev)
+            t_gw = torch.empty(cc.n_logical, dtype=torch.float32, device=dev)
+            t_ow = torch.empty(ng, g2, d2, dtype=torch.float32, device=dev)
+            t_out = torch.empty_like(t_idx)
+            t_args = (t_idx.data_ptr(), t_idx.numel(), t_cnt.data_ptr(), t_r2o.data_ptr(), t_o2r.data_ptr(),
+                      t_p2l.data_ptr(), ng, g2, d2, c2, p2, n_sms, t_by.data_ptr(), t_gw.data_ptr(), t_ow.data_ptr(),
+                      avail.data_ptr(), t_out.data_ptr(), None, 0, 5, stream)
+
+            def plan_cfg():
+                assert lib.lplb_plan(*t_args) == 0
+            row = {"indices": list(ci.indices.shape), "group_size": g2}
+            us = event_times_us(plan_cfg, 500, 50, torch)
+            row["one_launch_us_p50"], row["one_launch_us_p99"] = round(pct(us, 50), 2), round(pct(us, 99), 2)
+            assert lib.lplb_plan_set_cooperative(0) == 0
+            us = event_times_us(plan_cfg, 500, 50, torch)
+            row["chain_us_p50"], row["chain_us_p99"] = round(pct(us, 50), 2), round(pct(us, 99), 2)
+            assert lib.lplb_plan_set_cooperative(1) == 0
+            lp_timer = KernelTimer(lib, 100)
+            for _ in range(100):
+                lp_timer.arm()
+                assert lib.lplb_solve(t_cnt.data_ptr(), t_gw.data_ptr(), t_r2o.data_ptr(), t_p2l.data_ptr(), ng, g2, d2,
+                                      c2, l2 - c2 * d2, avail.data_ptr(), t_ow.data_ptr(), 0, 5, stream) == 0
+            row["lp_kernel_us_p50"] = round(pct(lp_timer.times_us(torch), 50), 2)
+            lp_timer.close()
+            per_cfg[name] = row
+        extras["per_config"] = per_cfg
 
         # Planner.run through the Python API, wall clock with a device sync (host overhead included)
         from lplb_amd import Planner
@@ -438,6 +533,33 @@ def main() -> None:
                     "sample": f"{len(cpu_us)} plans of the same v3_ep8_cube inputs in {args.cpu_seconds:.0f} s, "
                               f"scalar C restatement of the reference algorithm, host has {os.cpu_count()} CPUs",
                     "p99": round(pct(cpu_us, 99), 1)}
+    # The same plan on PyTorch CPU tensors (bincount / cumsum, dense fp32 LP, torch.linalg.cholesky, vectorised
+    # redirect), once with one thread and once with every host core: 20 warm-up + up to 200 timed plans each.
+    if args.cpu_seconds > 0:
+        from oracle import torch_plan
+        t_idx_h, t_counts_h = torch.from_numpy(idx_h), torch.from_numpy(counts_h)
+        t_p2l_h, t_o2r_h = torch.from_numpy(inp.phy2log), torch.from_numpy(o2r_host)
+        dense = torch_plan.DenseLp(cfg.r2o, C, n_fixed)
+
+        def torch_cpu_plan():
+            by = torch_plan.count_idx(t_idx_h, cfg.n_logical, n_sms)
+            shares, _, _ = torch_plan.solve(t_counts_h, dense, t_p2l_h, 1)
+            return torch_plan.map_idx(t_idx_h, shares, by, t_o2r_h, t_p2l_h, 1, C, P)
+        torch_rows = {}
+        for threads in (1, os.cpu_count() or 1):
+            torch.set_num_threads(threads)
+            for _ in range(20):
+                torch_cpu_plan()
+            samples = []
+            t_stop = time.perf_counter() + args.cpu_seconds / 2
+            while len(samples) < 200 and time.perf_counter() < t_stop:
+                t = time.perf_counter_ns()
+                torch_cpu_plan()
+                samples.append((time.perf_counter_ns() - t) / 1e3)
+            torch_rows[f"threads_{threads}"] = {"p50_us": round(pct(samples, 50), 1), "p99_us": round(pct(samples, 99), 1),
+                                                "plans": len(samples), "torch_num_threads": torch.get_num_threads()}
+        cpu_baseline["pytorch_cpu_restatement"] = torch_rows
+        cpu_baseline["host_cpus"] = os.cpu_count()
 
     line = {
         "metric": "p50 us per plan (histogram + LP solve + redirect), EP8 cube V3 shape",

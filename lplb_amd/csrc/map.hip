@@ -62,8 +62,10 @@ static size_t map_lds_bytes(int n_logical, int n_rep, int w, int k) {
 // code from the first load to the first barrier has no branch, which lets the compiler
 // count outstanding loads exactly: the tables are built from the small loads while the
 // index loads issued after them are still in flight.
-template <int K, bool WRAP, bool TAIL>
-__global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) {
+// SINGLE: a slice is at most one pass long (no second set of loads in flight, and the
+// registers that saves let twice as many waves stay resident).
+template <int K, bool WRAP, bool TAIL, bool SINGLE>
+__global__ __launch_bounds__(kMaxWaves *kWave, SINGLE ? 8 : 4) void redirect_indices(MapArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int kRec = rank_record_bytes(K);
   const int nl = a.n_logical, R = a.n_rep;
@@ -137,10 +139,11 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
         raw[c] = w0 + c * kWave + lane < end ? __builtin_nontemporal_load(src + c * kWave) : -1;
     }
   };
-  int64_t raw0[K], raw1[K];
+  int64_t raw0[K], raw1[SINGLE ? 1 : K];
   issue_loads(raw0, begin);
   // (without TAIL a slice of one pass loads that pass twice rather than branch here)
-  issue_loads(raw1, (TAIL || begin + pass_len < end) ? begin + pass_len : begin);
+  if constexpr (!SINGLE)
+    issue_loads(raw1, (TAIL || begin + pass_len < end) ? begin + pass_len : begin);
 
   // ---- tables ----
   for (int e = tid; e <= nl; e += nt)
@@ -224,8 +227,9 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
       original[c] = rt.original;
       set[c] = rt.rep;
     }
-    if (pass + 2 * pass_len < end)
-      issue_loads(raw, pass + 2 * pass_len);   // in flight during this pass and the next
+    if constexpr (!SINGLE)
+      if (pass + 2 * pass_len < end)
+        issue_loads(raw, pass + 2 * pass_len);   // in flight during this pass and the next
     // Phase A.
     ChunkSlot *slot[K];
 #pragma unroll
@@ -305,11 +309,16 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
     LPLB_MAP_STAMP(5 + 4 * PAR);
   };
 
-  for (int64_t pass = begin; pass < end; pass += 2 * pass_len) {
-    process(std::integral_constant<int, 0>{}, raw0, pass);
-    if (pass + pass_len >= end)
-      break;
-    process(std::integral_constant<int, 1>{}, raw1, pass + pass_len);
+  if constexpr (SINGLE) {
+    if (begin < end)
+      process(std::integral_constant<int, 0>{}, raw0, begin);
+  } else {
+    for (int64_t pass = begin; pass < end; pass += 2 * pass_len) {
+      process(std::integral_constant<int, 0>{}, raw0, pass);
+      if (pass + pass_len >= end)
+        break;
+      process(std::integral_constant<int, 1>{}, raw1, pass + pass_len);
+    }
   }
 
 #ifdef LPLB_PHASE_CLOCKS
@@ -323,14 +332,14 @@ __global__ __launch_bounds__(kMaxWaves *kWave) void redirect_indices(MapArgs a) 
 int g_force_waves = 0, g_force_k = 0;
 #endif
 
-template <int K, bool WRAP, bool TAIL>
+template <int K, bool WRAP, bool TAIL, bool SINGLE>
 static hipError_t launch_redirect_variant(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
   if (lds > 64 * 1024) {
-    const hipError_t err = allow_dynamic_lds(&redirect_indices<K, WRAP, TAIL>, 160 * 1024);
+    const hipError_t err = allow_dynamic_lds(&redirect_indices<K, WRAP, TAIL, SINGLE>, 160 * 1024);
     if (err != hipSuccess)
       return err;
   }
-  launch(redirect_indices<K, WRAP, TAIL>, grid, block, lds, s, a);
+  launch(redirect_indices<K, WRAP, TAIL, SINGLE>, grid, block, lds, s, a);
   return hipGetLastError();
 }
 template <int K, bool WRAP>
@@ -338,8 +347,12 @@ static hipError_t launch_redirect(const MapArgs &a, dim3 grid, dim3 block, size_
   // every slice a whole number of passes?  (the last slice may be shorter than the others)
   const int64_t pass_len = (int64_t)block.x * K;
   const bool whole = a.per % pass_len == 0 && a.n % pass_len == 0;
-  return whole ? launch_redirect_variant<K, WRAP, false>(a, grid, block, lds, s)
-               : launch_redirect_variant<K, WRAP, true>(a, grid, block, lds, s);
+  const bool single = a.per <= pass_len;
+  if (single)
+    return whole ? launch_redirect_variant<K, WRAP, false, true>(a, grid, block, lds, s)
+                 : launch_redirect_variant<K, WRAP, true, true>(a, grid, block, lds, s);
+  return whole ? launch_redirect_variant<K, WRAP, false, false>(a, grid, block, lds, s)
+               : launch_redirect_variant<K, WRAP, true, false>(a, grid, block, lds, s);
 }
 
 } // namespace lplb

@@ -166,3 +166,25 @@ def edge_flows(workload, probs, r2o, phy2log, n_group: int, n_per_var: int) -> n
     pw = w[np.asarray(phy2log).reshape(-1)].reshape(n_group, G, -1)
     dup = pw[:, :, :n_per_var * D].reshape(n_group, G, n_per_var, D).sum(2)
     return (1 - np.asarray(probs, dtype=np.float64).reshape(n_group, G, D)) * dup
+
+
+def compare_batch(workloads, got, r2o, phy2log, n_group: int, n_per_var: int, n_fixed: int, *,
+                  step_rule: int = 0, n_steps: int = 5):
+    """Checks a batch of independent solves against this oracle (fp32).  workloads int32
+    [N, n_logical], got fp32 [N, n_group, G, D].  Returns (largest edge-flow difference as a
+    fraction of the instance's token count, largest relative objective difference, number of
+    feasible (instance, group) pairs according to the oracle)."""
+    workloads = np.asarray(workloads)
+    got = np.asarray(got)
+    worst_flow = worst_obj = 0.0
+    n_ok = 0
+    for w, res in zip(workloads, got):
+        ref, _, ok = solve(w, r2o, phy2log, n_group, n_per_var, n_fixed, step_rule=step_rule, n_steps=n_steps)
+        n_ok += ok
+        args = (r2o, phy2log, n_group, n_per_var)
+        flow = np.abs(edge_flows(w, res, *args) - edge_flows(w, ref, *args)).max() / float(w.sum(dtype=np.float64))
+        obj_ref = rank_loads(w, ref, *args).max(axis=1)
+        obj = rank_loads(w, res, *args).max(axis=1)
+        worst_flow = max(worst_flow, float(flow))
+        worst_obj = max(worst_obj, float((np.abs(obj - obj_ref) / obj_ref).max()))
+    return worst_flow, worst_obj, n_ok

@@ -188,6 +188,31 @@ def test_count_and_redirect_random_shapes(cuda):
 
 
 # -------------------------------------------------------------------- solver
+
+def _why_flags_may_differ(wl, r2o, phy2log, n_group, C, n_fixed, step_rule=0):
+    """The feasibility test compares three quantities with fixed thresholds (minilp.cu:381-382):
+    the last step's d_max < 0.1, 0 <= x_M < 1e-4 and the residual < 0.05.  Two correct evaluations
+    of the same algorithm can only disagree on the flag of a group when one of them is within
+    rounding reach of its threshold.  Returns, per group, the quantities that lie within 10 % of
+    a threshold in the fp64 evaluation (for the lower bound 0 of x_M: |x_M| below 1e-5, the
+    absolute counterpart), or 'not finite'; an empty list means the flag is not in doubt."""
+    _, _, _, x, trace, resid = oracle.solve(wl, r2o, phy2log, n_group, C, n_fixed, precision=64, details=True,
+                                            step_rule=step_rule)
+    out = []
+    for g in range(n_group):
+        d_max, x_m, res = float(trace[g, -1, 0]), float(x[g, -1]), float(resid[g])
+        near = []
+        if not np.isfinite([d_max, x_m, res]).all():
+            near.append("not finite")
+        if abs(d_max - 0.1) <= 0.01:
+            near.append(f"d_max={d_max:.4g}")
+        if abs(x_m - 1e-4) <= 1e-5 or abs(x_m) <= 1e-5:
+            near.append(f"x_M={x_m:.3g}")
+        if abs(res - 0.05) <= 0.005:
+            near.append(f"residual={res:.4g}")
+        out.append(near)
+    return out
+
 def _compare_solve(shape, phy2log, workload, res, gw, avail, step_rule=0, n_steps=5):
     o_res, o_gw, o_avail = oracle.solve(workload, shape.r2o, phy2log, shape.n_group, shape.C, shape.n_fixed,
                                         step_rule=step_rule, n_steps=n_steps)
@@ -270,6 +295,7 @@ def test_solve_adversarial_distributions(cuda, topo):
         return rng.multinomial(int(rng.choice([1000, 65536, 1 << 22])), p / p.sum()).astype(np.int32)
 
     flags_differ = checked = 0
+    skipped = []
     worst = [0.0, 0.0]
     for kind in ("zipf1", "zipf2", "lognorm", "near_uniform", "sparse", "one_hot"):
         for _ in range(8):
@@ -283,10 +309,15 @@ def test_solve_adversarial_distributions(cuda, topo):
             o64, o_gw, o_avail = oracle.solve(wl, r2o, phy2log, shape.n_group, shape.C, shape.n_fixed, precision=64)
             np.testing.assert_array_equal(gw.cpu().numpy().reshape(-1), o_gw)
             if int(avail[0]) != o_avail:
+                # allowed only where the fp64 evaluation itself sits on a threshold
+                why = _why_flags_may_differ(wl, r2o, phy2log, shape.n_group, shape.C, shape.n_fixed)
+                assert any(why), f"{topo}/{kind}: feasible on GPU {int(avail[0])}, fp64 oracle {o_avail}, no quantity near a threshold"
+                skipped.append(f"{kind}: flags differ ({int(avail[0])} vs {o_avail}), {why}")
                 flags_differ += 1
                 continue
             if o_avail != shape.n_group:
                 assert np.all(res == 0.5)
+                skipped.append(f"{kind}: infeasible in both evaluations, neutral split returned")
                 continue
             args = (r2o, phy2log, shape.n_group, shape.C)
             flow = np.abs(oracle.edge_flows(wl, res, *args) - oracle.edge_flows(wl, o64, *args)).max() / float(wl.sum())
@@ -294,8 +325,11 @@ def test_solve_adversarial_distributions(cuda, topo):
             worst = [max(worst[0], flow), max(worst[1], float((np.abs(obj - obj64) / obj64).max()))]
             checked += 1
     print(f"{topo}: {checked} compared, worst flow {worst[0]:.1e} objective {worst[1]:.1e}, feasibility differs in {flags_differ}")
+    for line in skipped:
+        print("  not compared:", line)
     assert worst[0] <= FLOW_TOL and worst[1] <= OBJ_RTOL
-    assert flags_differ <= 2 and checked >= 40
+    # of 48 inputs per topology: at most 2 threshold cases, at most 8 without flows to compare
+    assert flags_differ <= 2 and len(skipped) <= 8 and checked >= 40
 
 
 @pytest.mark.gpu
@@ -315,6 +349,7 @@ def test_solve_random_topologies(cuda, G, D, C, n_group):
     assert (shape.C, shape.n_fixed) == (C, per_rank - D * C)
     solver = solver_for(shape)
     compared = 0
+    skipped = []
     for trial in range(6):
         # any assignment of logical experts to slots is a legal phy2log layout: originals are a
         # permutation, replica slot (rank, c*D+d) copies slot c*D+d of rank r2o[rank][d]
@@ -335,14 +370,67 @@ def test_solve_random_topologies(cuda, G, D, C, n_group):
         res = res.cpu().numpy()
         o64, o_gw, o_avail = oracle.solve(wl, r2o, phy2log, n_group, C, shape.n_fixed, precision=64)
         np.testing.assert_array_equal(gw.cpu().numpy().reshape(-1), o_gw)
-        if int(avail[0]) != o_avail or o_avail != n_group:
-            continue                        # a flag on the edge of a threshold; counted below
+        if int(avail[0]) != o_avail:
+            # allowed only where the fp64 evaluation itself sits on a threshold
+            why = _why_flags_may_differ(wl, r2o, phy2log, n_group, C, shape.n_fixed)
+            assert any(why), f"trial {trial}: feasible on GPU {int(avail[0])}, fp64 oracle {o_avail}, no quantity near a threshold"
+            skipped.append(f"trial {trial}: flags differ ({int(avail[0])} vs {o_avail}), {why}")
+            continue
+        if o_avail != n_group:
+            # some group infeasible in both: it must carry the neutral split, the others are compared below
+            failed = [g for g in range(n_group) if np.all(o64[g] == 0.5)]
+            assert len(failed) == n_group - o_avail and all(np.all(res[g] == 0.5) for g in failed), trial
+            skipped.append(f"trial {trial}: {len(failed)} of {n_group} groups infeasible in both evaluations")
         args = (r2o, phy2log, n_group, C)
         flow = np.abs(oracle.edge_flows(wl, res, *args) - oracle.edge_flows(wl, o64, *args)).max() / float(wl.sum())
         obj, obj64 = (oracle.rank_loads(wl, x, *args).max(axis=1) for x in (res, o64))
         assert flow <= FLOW_TOL and np.all(np.abs(obj - obj64) <= OBJ_RTOL * obj64), (trial, flow)   # a group may be empty
         compared += 1
-    assert compared >= 4
+    for line in skipped:
+        print("  note:", line)
+    # six draws per topology: at most one may end on a threshold
+    assert compared >= 5 and sum("flags differ" in line for line in skipped) <= 1
+
+
+def test_solve_window_rule_chaos_regression(cuda):
+    """A legal input on which the reference's step rule (d_max over the last 32 columns only,
+    minilp.cu:355-359) lets the iterates leave [0, 1] by far: 64 ranks on one random replica
+    permutation, 4 194 305 tokens (tests/golden/window_chaos_ring64.json, written by
+    make_window_chaos_case.py).  The exact-arithmetic iteration returns shares between -84 and
+    +49 and still reports feasible.  In that regime rounding is amplified: the dense fp32
+    evaluation ends 2.4e-3 of the tokens away from the fp64 one, beyond the 1e-4 parity
+    tolerance, so the tolerance cannot hold against the fp32 oracle here.  Expected
+    classification: window-rule chaos; the GPU result (fp64 normal-equation core) is feasible
+    like both oracles and lies closer to the fp64 evaluation than the fp32 evaluation does."""
+    import json
+    from pathlib import Path
+    case = json.loads((Path(__file__).parent / "golden" / "window_chaos_ring64.json").read_text())
+    r2o = np.asarray(case["r2o"], np.int32).reshape(64, 1)
+    phy2log, wl = np.asarray(case["phy2log"], np.int32), np.asarray(case["workload"], np.int32)
+    shape = Shape(r2o, 64, 64, 128)
+    solver = solver_for(shape)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    res, gw = solver.solve(dev(wl.reshape(1, 64, 1), cuda), dev(r2o, cuda), dev(phy2log, cuda), avail)
+    res = res.cpu().numpy()
+    o64, o_gw, ok64 = oracle.solve(wl, r2o, phy2log, 1, 1, 0, precision=64)
+    o32, _, ok32 = oracle.solve(wl, r2o, phy2log, 1, 1, 0, precision=32)
+    np.testing.assert_array_equal(gw.cpu().numpy().reshape(-1), o_gw)
+    assert int(avail[0]) == ok64 == ok32 == 1
+    assert o64.min() < -50 and o64.max() > 40          # the classification: shares far outside [0, 1]
+    args = (r2o, phy2log, 1, 1)
+    total = float(wl.sum())
+    flows = {k: oracle.edge_flows(wl, v, *args) for k, v in (("gpu", res), ("f64", o64), ("f32", o32))}
+    gpu_vs_64 = np.abs(flows["gpu"] - flows["f64"]).max() / total
+    f32_vs_64 = np.abs(flows["f32"] - flows["f64"]).max() / total
+    print(f"window chaos: GPU {gpu_vs_64:.2e} of the tokens from fp64, fp32 oracle {f32_vs_64:.2e}")
+    assert f32_vs_64 > FLOW_TOL              # the fp32 evaluation itself is outside the tolerance
+    assert gpu_vs_64 < f32_vs_64 and gpu_vs_64 <= 1e-3
+    # with the step taken over all columns the same input is tame and the usual bar holds
+    solver.step_rule = 1
+    avail.zero_()
+    res1, gw1 = solver.solve(dev(wl.reshape(1, 64, 1), cuda), dev(r2o, cuda), dev(phy2log, cuda), avail)
+    _compare_solve(shape, phy2log, wl, res1.cpu().numpy(), gw1.cpu().numpy(), int(avail[0]), step_rule=1)
+    assert 0 <= res1.min() and res1.max() <= 1
 
 
 def test_solve_fallback_and_counter(cuda):
@@ -382,6 +470,27 @@ def test_solve_batched_matches_single(cuda):
         single, gw = solver.solve(dev(counts[i].reshape(1, shape.G, shape.L), cuda), r2o, p2l, avail)
         assert torch.equal(single[0], batched[i, 0]) and torch.equal(gw, gws[i])
         _compare_solve(shape, inp.phy2log, counts[i], batched[i].cpu().numpy(), gws[i].cpu().numpy(), 1)
+
+
+def test_solve_batched_throughput_sweep_all_2048_against_oracle(cuda):
+    """The solver half of the throughput sweep: 2048 independent V3 / EP8-cube count vectors in one
+    launch (one block per LP in the reference, csrc/plugin.cpp:559-565; here four LPs per wave from
+    1536 LPs on).  Every one of the 2048 results is held against the fp32 oracle."""
+    inp = synth.make_inputs("v3_ep8_cube", tokens=8)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    counts = synth.sweep_counts(2048)
+    solver = solver_for(shape)
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    res, gws = solver.solve_batched(dev(counts.reshape(2048, 1, shape.G, shape.L), cuda), dev(shape.r2o, cuda),
+                                    dev(inp.phy2log, cuda), avail, want_global=True)
+    torch.cuda.synchronize()
+    flow, obj, n_ok = oracle.compare_batch(counts, res.cpu().numpy(), shape.r2o, inp.phy2log, 1, shape.C, shape.n_fixed)
+    print(f"2048 LPs: worst flow diff {flow:.2e} of the tokens, worst objective diff {obj:.2e}, feasible {n_ok}")
+    assert flow <= FLOW_TOL and obj <= OBJ_RTOL
+    assert int(avail[0]) == n_ok == 2048
+    for i in (0, 1000, 2047):
+        np.testing.assert_array_equal(gws[i].cpu().numpy().reshape(-1), oracle.normalise(counts[i]))
 
 
 def _shifted_ring(g, shifts):

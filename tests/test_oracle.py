@@ -329,3 +329,56 @@ def test_solver_fp32_tracks_fp64():
         r32 = oracle.solve(inp.global_counts, c.r2o, inp.phy2log, 1, s.C, s.n_fixed)[0]
         r64 = oracle.solve(inp.global_counts, c.r2o, inp.phy2log, 1, s.C, s.n_fixed, precision=64)[0]
         assert np.abs(r32 - r64).max() < 1e-3
+
+
+def test_window_rule_chaos_fixture_is_what_it_says():
+    """tests/golden/window_chaos_ring64.json: under the reference's step rule (d_max over the last 32
+    columns, minilp.cu:355-359) the exact iteration leaves [0, 1] by far, stays 'feasible', keeps
+    A x = b (x_o + x_r - x_M = 1 on every edge) -- and its fp32 evaluation drifts beyond the parity
+    tolerance; with the maximum over all columns the same input is tame."""
+    case = json.loads((Path(__file__).parent / "golden" / "window_chaos_ring64.json").read_text())
+    r2o = np.asarray(case["r2o"], np.int32).reshape(64, 1)
+    phy2log, wl = np.asarray(case["phy2log"], np.int32), np.asarray(case["workload"], np.int32)
+    r64, _, ok64, x, _, _ = oracle.solve(wl, r2o, phy2log, 1, 1, 0, precision=64, details=True)
+    r32, _, ok32 = oracle.solve(wl, r2o, phy2log, 1, 1, 0)
+    assert ok64 == ok32 == 1 and r64.min() < -50 and r64.max() > 40
+    x = x[0]
+    np.testing.assert_allclose(x[:64] + x[64:128] - x[-1], 1.0, atol=1e-9)
+    args = (r2o, phy2log, 1, 1)
+    drift = np.abs(oracle.edge_flows(wl, r32, *args) - oracle.edge_flows(wl, r64, *args)).max() / wl.sum()
+    assert 1e-4 < drift < 1e-2
+    tame = oracle.solve(wl, r2o, phy2log, 1, 1, 0, precision=64, step_rule=1)[0]
+    assert 0 <= tame.min() and tame.max() <= 1
+
+
+@pytest.mark.parametrize("name", ["cpu_ref_ep8", "v3_ep8_cube", "ep16_hypercube"])
+def test_torch_restatement_agrees_with_the_c_restatement(name):
+    """oracle/torch_plan.py (the multi-threaded CPU baseline that bench.py times) against
+    lplb_oracle.c: histogram and redirect bit for bit, LP shares to fp32 rounding."""
+    import torch
+    from oracle import torch_plan
+    inp = synth.make_inputs(name, mask_fraction=0.05, tokens=600)
+    c = inp.cfg
+    s = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    idx = torch.from_numpy(inp.indices)
+    by = torch_plan.count_idx(idx, c.n_logical, 7)
+    want_by = oracle.count_idx(inp.indices, c.n_logical, 7)
+    np.testing.assert_array_equal(by.numpy(), want_by)
+    lp = torch_plan.DenseLp(c.r2o, s.C, s.n_fixed)
+    dupw, b, a, cost = oracle.build_lp(inp.global_counts, c.r2o, inp.phy2log, s.n_group, 0, s.C, s.n_fixed)
+    gw = torch.from_numpy(oracle.normalise(inp.global_counts))
+    A, bb = lp.build(gw, torch.from_numpy(inp.phy2log.reshape(s.n_group, s.G, s.P)[0].astype(np.int64)))
+    np.testing.assert_allclose(A.numpy(), a, atol=2e-6)
+    np.testing.assert_allclose(bb.numpy(), b, atol=1e-6)
+    np.testing.assert_array_equal(lp.c.numpy(), cost)
+    res, gw2, n_ok = torch_plan.solve(torch.from_numpy(inp.global_counts), lp, torch.from_numpy(inp.phy2log), s.n_group)
+    want, want_gw, want_ok = oracle.solve(inp.global_counts, c.r2o, inp.phy2log, s.n_group, s.C, s.n_fixed)
+    np.testing.assert_array_equal(gw2.numpy(), want_gw)
+    assert n_ok == want_ok == s.n_group
+    args = (c.r2o, inp.phy2log, s.n_group, s.C)
+    flow = np.abs(oracle.edge_flows(inp.global_counts, res.numpy(), *args) - oracle.edge_flows(inp.global_counts, want, *args))
+    assert flow.max() <= 1e-3 * inp.global_counts.sum()     # two fp32 evaluations of an ill-conditioned iteration
+    out = torch_plan.map_idx(idx, torch.from_numpy(want), by, torch.from_numpy(s.o2r), torch.from_numpy(inp.phy2log),
+                             s.n_group, s.C, s.P)
+    want_out = oracle.map_idx(inp.indices, want, want_by, s.o2r, inp.phy2log, s.n_group, s.C, s.P)
+    np.testing.assert_array_equal(out.numpy(), want_out)
