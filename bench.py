@@ -421,6 +421,7 @@ def main() -> None:
         assert lib.lplb_plan_set_cooperative(1) == 0
         timeouts = ctypes.c_int(-1)
         assert lib.lplb_plan_sync_timeouts(ctypes.byref(timeouts)) == 0 and timeouts.value == 0, timeouts.value
+        extras["plan_waits_that_ran_out"] = timeouts.value
 
         # the same plan replayed from a HIP graph (8 plans per graph): GPU-side cost without launch overhead
         per_graph = 8

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 3
+#define LPLB_ABI_VERSION 4
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -181,13 +181,18 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  *   out              int64 [n_elements], out (see lplb_map_idx)
  *   physical_counts  int32 [n_physical] or NULL, out (see lplb_map_idx)
  *
- * The one-launch form keeps its counters in a per-device array of the library, one
- * block for each of the first eight streams that plan (further streams get the
- * chain).  Launches that share a block must not overlap in time, which stream order
- * guarantees; the exception is a graph captured on one stream and replayed
- * concurrently on several.  A launch takes up to a quarter of the GPU's CUs (plus one per four EP groups) and its
- * workgroups wait for each other, so at most three plans may execute at the same
- * time on a device (see lplb_plan_set_cooperative).
+ * The one-launch form: its workgroups wait for each other, so the whole grid has to be
+ * resident on the GPU.  The library admits a launch only if the grid fits (occupancy
+ * query) beside the one-launch plans that are still executing, of which it keeps
+ * track per stream (eight streams per device at a time; it asks the runtime whether
+ * those streams still have work pending, it never waits); otherwise the call runs the
+ * chain, with identical results.  A plan captured into a graph keeps its share of the GPU reserved
+ * from then on (its replays are invisible to the library).  Launches on one stream never overlap; the exception the
+ * library cannot see is a graph captured on one stream and replayed concurrently on
+ * several (see lplb_plan_set_cooperative).  Every wait inside the kernel is bounded; if one
+ * runs out (lplb_plan_sync_timeouts), the launch still completes with a valid but
+ * unbalanced result: the tokens of the affected slices go to their experts' original
+ * slots, avail_num is left unchanged and physical_counts, if given, is filled with -1.
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -240,10 +245,25 @@ int lplb_plan_set_cooperative(int enabled);
  * No counterpart in the reference.  The workgroups of the one-launch plan wait
  * for each other with a bounded number of polls; *count receives how many waits
  * ran out on the current device since the library was loaded (0 in a healthy
- * run; a plan with a wait that ran out has undefined output).  Synchronous:
- * copies a few ints from the device.
+ * run; what a plan with such a wait returns is described at lplb_plan).
+ * Synchronous: copies a few ints from the device.
  */
 int lplb_plan_sync_timeouts(int *count);
+
+/*
+ * No counterpart in the reference.  *count receives how many lplb_plan /
+ * lplb_plan_noalloc calls of this process ran as one kernel launch (the others ran
+ * the chain of kernels).  For callers and tests that want to know which form they got.
+ */
+int lplb_plan_one_launch_count(long long *count);
+
+/*
+ * Test hook, no counterpart in the reference.  The next plan that runs as one launch
+ * waits for extra_slices_expected more slices than its grid has (so the wait cannot be
+ * met) and gives up after max_polls polls instead of millions (0 = the default bound).
+ * Every kernel still ends normally; the call exists to exercise the give-up path.
+ */
+int lplb_plan_inject_fault(int extra_slices_expected, int max_polls);
 
 #ifdef __cplusplus
 }

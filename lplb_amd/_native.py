@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1
@@ -40,6 +40,8 @@ _SIGNATURES = {
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_plan_set_cooperative": (_i, [_i]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
+    "lplb_plan_one_launch_count": (_i, [_vp]),
+    "lplb_plan_inject_fault": (_i, [_i, _i]),
     "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "lplb_plan_noalloc": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
 }
@@ -88,6 +90,13 @@ def plan_sync_timeouts() -> int:
     """Waits between workgroups of the one-launch plan that ran out on the current device (0 when healthy)."""
     count = ctypes.c_int(-1)
     _check(load().lplb_plan_sync_timeouts(ctypes.byref(count)))
+    return count.value
+
+
+def plan_one_launch_count() -> int:
+    """Plans of this process that ran as one kernel launch (the others ran the chain of kernels)."""
+    count = ctypes.c_longlong(-1)
+    _check(load().lplb_plan_one_launch_count(ctypes.byref(count)))
     return count.value
 
 

@@ -223,22 +223,28 @@ template <int N> __device__ inline int row_shr(int v) {
 template <int CTRL> __device__ inline int dpp_int(int v) {
   return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
 }
-// Sum over each group of K adjacent lanes (K = 1, 2, 4 or 8; every lane gets its group's sum).
+// Sum over each group of K adjacent lanes (K = 1, 2, 4, 8 or 16; every lane gets its group's sum).
 template <int K> __device__ inline int group_sum(int v) {
   if constexpr (K >= 2) v += dpp_int<0xB1>(v);    // quad_perm [1,0,3,2]
   if constexpr (K >= 4) v += dpp_int<0x4E>(v);    // quad_perm [2,3,0,1]
   if constexpr (K >= 8) v += dpp_int<0x141>(v);   // row_half_mirror
+  if constexpr (K >= 16) v += dpp_int<0x140>(v);  // row_mirror
   return v;
 }
-// Sum of the lanes before this one in its group of K adjacent lanes (pos = lane % K).
+// Sum of the lanes before this one in its group of K adjacent lanes (pos = lane % K):
+// an inclusive scan in log2(K) shift-and-add steps, minus the lane's own value.
 template <int K> __device__ inline int group_exclusive_scan(int v, int pos) {
-  int acc = 0;
-  static_for<K - 1>([&](auto jc) {
-    constexpr int j = decltype(jc)::value + 1;
-    const int from_left = row_shr<j>(v);
-    acc += pos >= j ? from_left : 0;
-  });
-  return acc;
+  int acc = v;
+  if constexpr (K >= 2) { const int t = row_shr<1>(acc); acc += pos >= 1 ? t : 0; }
+  if constexpr (K >= 4) { const int t = row_shr<2>(acc); acc += pos >= 2 ? t : 0; }
+  if constexpr (K >= 8) { const int t = row_shr<4>(acc); acc += pos >= 4 ? t : 0; }
+  if constexpr (K >= 16) { const int t = row_shr<8>(acc); acc += pos >= 8 ? t : 0; }
+  return acc - v;
 }
+
+// Ranking record of one (wave, replicated set) when a slice is a single pass: K chunk
+// slots; from four slots on padded to an odd multiple of 16 bytes (a record of 64, 128 or
+// 256 bytes would put every set into the same LDS banks).
+constexpr int rank_record_bytes_single(int k) { return k * (int)sizeof(ChunkSlot) + (k >= 4 ? 16 : 0); }
 
 } // namespace lplb

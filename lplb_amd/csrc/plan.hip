@@ -5,179 +5,211 @@
 // Chain: the three entry points' kernels one after the other (histogram, scan,
 // LP, redirect).  With the global counts supplied the LP does not depend on this
 // GPU's histogram: it is enqueued first and the histogram launch does not wait for
-// it (it still starts after everything the LP launch waited for).  Running the LP
-// as a parallel branch of a captured HIP graph (side stream + events) was measured
-// and rejected: 24.6 us per plan against 20.0 us for the plain chain in the graph.
+// it (it still starts after everything the LP launch waited for).
 //
-// One launch (plan_in_one_launch): for batches of up to 64 slices of 8192 indices
-// (4096 with 512-thread workgroups) and LP shapes whose registers fit beside a 512-
-// or 1024-thread workgroup.  Every
-// kernel boundary of the chain costs 3-5 us on this GPU although the kernels have
-// 1-3 us of work, and the LP (8 us, one wave) sits on the critical path.  Here one
-// workgroup per slice and one more per four LPs run side by side in a single grid:
-//   slice workgroup: load indices -> per-wave LDS histograms -> publish the slice's
-//     histogram row -> wait until all rows are there -> add up the rows (totals and
-//     counts before this slice) -> tables and per-wave starting ordinals -> wait for
-//     the LP's shares -> redirect and store;
-//   LP workgroup: (own-histogram mode: wait for the rows, add them up) -> solve ->
-//     publish the shares.
-// What crosses workgroups (rows, shares, three counters) is written and read with
-// agent-scope atomics, which go through the XCD's L2 to memory; nothing else is
-// shared, so no cache write-back or invalidate is needed.  The grid is far smaller
-// than the GPU (at most 72 workgroups on 256 CUs), so all workgroups are resident
-// and the waits end; each wait is bounded all the same, and a wait that runs out is
-// counted (lplb_plan_sync_timeouts) instead of hanging the GPU.  The counters live
-// in a per-device array of this library, one block per stream (the first eight streams
-// that run a plan; further streams get the chain); the last workgroup to leave
-// clears its block, so a captured launch can be replayed.  Launches that share a
-// block must not overlap in time: that holds for one stream's launches, not for
-// graphs captured on one stream and replayed concurrently on several; and no more
-// than three plans may execute at the same time on a device -- callers outside
-// these limits switch this path off with lplb_plan_set_cooperative(0).
+// One launch (plan_in_one_launch): every kernel boundary of the chain costs 3-5 us
+// on this GPU although the kernels have 1-8 us of work, and the LP (8 us, one wave)
+// sits on the critical path.  Here the LP workgroups (one per four LPs, first in the
+// grid) and one workgroup per slice of the indices run side by side in a single grid:
+//   slice workgroup: load indices (once; they stay in registers) -> LDS histogram and
+//     per-chunk bitmaps of the replicated sets -> add the histogram to the batch's
+//     totals and publish the slice's counts of the replicated sets -> wait until all
+//     slices have -> tokens of each set before this slice and in the batch -> ordinals
+//     and hashes -> wait for the LP's shares -> choose original or replica, store;
+//   LP workgroup: (own-histogram mode: wait for the totals ->) solve -> publish the shares.
+// What crosses workgroups is written and read with agent-scope atomics (plan_sync.h).
+// The workgroups wait for each other, so the whole grid has to be resident: its size is
+// bounded by what the occupancy query says fits the GPU, and the host admits a launch
+// only while the plans still executing leave room for it (it asks the runtime whether the
+// streams that planned last still have work pending; it never waits); everything else
+// runs as the chain.  Every wait
+// is bounded all the same.  A wait that runs out is counted and the launch degrades
+// in a defined way: every token of the affected slices goes to its expert's original
+// slot (which needs nothing from other workgroups), the feasible-LP counter is left
+// alone and physical_counts, if asked for, is filled with -1.
 #include "map_kernel.h"
+#include "plan_sync.h"
 #include "solve_kernel.h"
 #include <atomic>
 #include <mutex>
+#include <stdio.h>
 
 namespace lplb {
 
-constexpr int kMaxSlices = 64;         // slice workgroups of the one-launch plan
-constexpr int kChunksPerWave = 8;     // its longest slice: 8 chunks of 64 indices per wave
-constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has 4 KB of static LDS besides
-constexpr int kMaxPolls = 1 << 22;    // a few seconds of polling before a wait gives up
+constexpr int kPreferredSlices = 64;   // short batches: slices of 1024, 2048, ... indices while this many cover them
+constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has static LDS besides
+constexpr int kDefaultMaxPolls = 1 << 22;   // a few seconds of polling before a wait gives up
 // LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP
 // wave is bound by instruction issue, so a fifth LP on the same CU would slow two of them
 // down (8 LPs in one workgroup: 17.0 us per plan against 13.5 us).  Batches with more
 // groups get more LP workgroups.
 constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 
-// [0] slices whose histogram row is published, [1] workgroups that have left,
-// [3] waits that ran out since the library was loaded; from kSharesAt on, the LP's
-// shares as 8-byte words (1 << 32) | float bits, 0 = not there yet.
-// From kTotalsAt on (own-histogram mode), one 8-byte word per logical expert: the
-// batch's tokens of that expert in the high half and the number of slices that have
-// added theirs in the low half -- one atomic add per slice and expert delivers both,
-// so the reader needs no second round trip for a "done" counter.
-constexpr int kSharesAt = 16, kMaxShares = 1024;
-constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024;
-// One such block per stream that has run a plan (the compute stream, a warm-up
-// stream, a graph-capture stream ...), so that plans enqueued on different streams
-// do not share counters.  A launch takes at most a quarter of the CUs (+ 8): up to three
-// plans that really execute at the same time are all resident; with four or more,
-// workgroups could wait for workgroups that cannot start.
-constexpr int kSlotInts = kTotalsAt + 2 * kMaxTotals, kSyncSlots = 8;
+// One block of these per stream that plans (kSyncSlots of them per device):
+//   [kArrivedAt ..] slices that have published their counts (striped), [kLeftStripesAt ..] and
+//   [kLeftAt] workgroups that need nothing from the others any more (see leave());
+//   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits, tag 0 = not
+//   there yet, 1 = valid, 2 = there will be none;
+//   from kTotalsAt: partial histograms of the batch, [copy][n_logical] 8-byte words with the
+//   tokens in the high half and the number of slices that have contributed in the low half
+//   (one atomic add delivers both, so whoever polls the words needs no second round trip
+//   for a "done" counter).  Slice s adds its histogram to copy s % n_copies: updates of one
+//   address queue up behind each other, about 35 ns each, so one copy per 16 slices (at most
+//   kTotalCopies); whoever needs the batch's tokens per expert adds the copies up.
+// The last workgroup to leave clears the block, so a captured launch can be replayed.
+constexpr int kLeftAt = 1;
+// ... and one that is never cleared: waits that ran out since the library was loaded
+constexpr int kTimeoutsAt = 4;
+constexpr int kArrivedAt = 16;      // kArrivalStripes words, one 64-byte line
+constexpr int kLeftStripesAt = 32;  // kArrivalStripes words: workgroups that have left, first level
+constexpr int kSharesAt = 48, kMaxShares = 1024;
+constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024, kTotalCopies = 16;
+constexpr int kSlotInts = kTotalsAt + 2 * kTotalCopies * kMaxTotals, kSyncSlots = 8;
 static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
 static std::atomic<bool> g_cooperative{true};   // any thread may flip it while others plan
+static std::atomic<long long> g_one_launch_plans{0};
+// Test hook (lplb_plan_inject_fault): the next one-launch plan expects this many slices
+// more than its grid has and gives up after this many polls.
+static std::atomic<int> g_fault_extra_slices{0}, g_fault_max_polls{0};
 
 struct PlanArgs {
   const int64_t *idx;
   int64_t n, per;
   int n_slices, n_lp_workgroups;
+  int n_copies;          // partial histograms of the batch: a power of two, at most kTotalCopies
+  int expected_slices;   // = n_slices unless a fault is injected
+  int max_polls;
   const int32_t *o2r, *phy2log;
-  int32_t *rows;     // [n_slices][n_logical] per-slice histograms, exchanged between workgroups
+  int32_t *rows;     // [n_slices << row_shift] per slice: its tokens of each replicated set
+  int row_shift;
   int32_t *totals;   // [n_logical] this GPU's tokens per expert, out
   int64_t *out;
   int32_t *physical_counts;   // [n_ranks * P] tokens per physical expert, or null
+  int32_t *avail;
   RedirectShape sh;
-  SolveArgs solve;   // result = the shares (o_weight); workload is replaced by totals if local_counts
+  int n_rep;
+  uint32_t magic_L, magic_cd, magic_D, magic_G;   // fast_div_magic of L, C * D, D, G
+  SolveArgs solve;   // result = the shares (o_weight); workload is replaced by the totals if local_counts
   int local_counts;
   int *sync;
 };
 
-__device__ inline int agent_load(const int *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ inline void agent_store(int *p, int v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// One lane polls *word until it reaches `target`; a wait that runs out is counted.
-// Afterwards this CU's L1 and this XCD's L2 drop what they hold of other XCDs'
-// memory, so that the plain (batched) loads that follow the workgroup barrier see
-// what the other workgroups wrote through to memory before they counted up.
-// (Agent-scope atomic loads would see it too, but the compiler issues those one
-// at a time: 16 of them cost 5 us.)
-__device__ inline void wait_for(int *sync, int word, int target) {
-  int polls = 0;
-  while (agent_load(sync + word) < target && ++polls < kMaxPolls)
-    __builtin_amdgcn_s_sleep(2);
-  if (polls >= kMaxPolls)
-    __hip_atomic_fetch_add(sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-}
-// rows[r][e] summed over r = first, first + step, ...: all rows (t) and those before
-// slice `pid` (before).
-__device__ inline void add_up_rows(const int32_t *rows, int n_rows, int nl, int e, int first, int step, int pid,
-                                   int32_t &t, int32_t &before) {
-  t = 0;
-  before = 0;
-  constexpr int kInFlight = 16;   // loads issued before the first is used (clamped addresses, masked values)
-  for (int r0 = first; r0 < n_rows; r0 += kInFlight * step) {
-    int32_t v[kInFlight];
-#pragma unroll
-    for (int k = 0; k < kInFlight; ++k)
-      v[k] = rows[(int64_t)min(r0 + k * step, n_rows - 1) * nl + e];
-#pragma unroll
-    for (int k = 0; k < kInFlight; ++k) {
-      const int r = r0 + k * step;
-      t += r < n_rows ? v[k] : 0;
-      before += r < pid ? v[k] : 0;
+// A wait ran out: count it (the workgroup also says so when it leaves).
+__device__ inline void give_up(const PlanArgs &a) { agent_add(a.sync + kTimeoutsAt, 1); }
+
+// Called by a whole workgroup when it needs nothing from the others any more.  The last of
+// the grid's workgroups to get here adds the feasible LPs to the caller's counter (unless a
+// wait ran out) and clears the block for the next launch (which starts after this kernel
+// has ended, so the clearing stores need no wait of their own).
+// Who is last is counted in two levels (updates of one address queue up, about 35 ns each):
+// the last of the workgroups that share a stripe counts for the stripe, the last stripe is
+// last.  What the last one has to know travels in the counters themselves: bits 0-11 count
+// workgroups or stripes, bits 12-23 those of them in which a wait ran out, bits 24-31 feasible LPs.
+// gave_up / feasible: LDS words of this workgroup, read after its waves have met.
+__device__ inline void leave(const PlanArgs &a, int n_shares, const int *gave_up, const int *feasible) {
+  __shared__ int last_to_leave, summary;
+  const int nl = a.sh.n_logical;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int n_workgroups = a.n_slices + a.n_lp_workgroups;
+    const int stripe = blockIdx.x % kArrivalStripes;
+    const int in_stripe = (n_workgroups - stripe + kArrivalStripes - 1) / kArrivalStripes;
+    const int mine = 1 + ((*gave_up ? 1 : 0) << 12) + (*feasible << 24);
+    const int of_stripe = agent_add(a.sync + kLeftStripesAt + stripe, mine) + mine;
+    last_to_leave = 0;
+    if ((of_stripe & 0xfff) == in_stripe) {
+      const int up = 1 + (((of_stripe >> 12) & 0xfff ? 1 : 0) << 12) + (of_stripe & 0xff000000);
+      const int all = agent_add(a.sync + kLeftAt, up) + up;
+      last_to_leave = (all & 0xfff) == min(n_workgroups, kArrivalStripes);
+      summary = all;
     }
   }
-}
-
-// Called by a whole workgroup when it is done.  The last of the grid's workgroups
-// to leave clears the counters and the shares for the next launch.
-__device__ inline void leave(int *sync, int n_workgroups, int n_shares, int n_totals) {
-  __shared__ int last_to_leave;
-  if (threadIdx.x == 0)
-    last_to_leave =
-        __hip_atomic_fetch_add(sync + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_workgroups - 1;
   __syncthreads();
   if (!last_to_leave)
     return;
-  unsigned long long *shares = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
+#ifdef LPLB_PHASE_CLOCKS
+  if (a.solve.clocks && threadIdx.x == 0)
+    a.solve.clocks[112] = wall_clock64();
+#endif
+  const bool failed = ((summary >> 12) & 0xfff) != 0;
+  unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
+  unsigned long long *totals = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt);
+  for (int i = threadIdx.x; i < a.n_copies * nl; i += blockDim.x)
+    agent_store(totals + i, 0ull);
   for (int i = threadIdx.x; i < n_shares; i += blockDim.x)
-    __hip_atomic_store(shares + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  for (int i = threadIdx.x; i < 2 * n_totals; i += blockDim.x)
-    agent_store(sync + kTotalsAt + i, 0);
+    agent_store(shares + i, 0ull);
+  if (threadIdx.x < kArrivalStripes) {
+    agent_store(a.sync + kArrivedAt + threadIdx.x, 0);
+    agent_store(a.sync + kLeftStripesAt + threadIdx.x, 0);
+  }
+  if (failed && a.physical_counts)
+    for (int i = threadIdx.x; i < a.sh.n_ranks * a.sh.P; i += blockDim.x)
+      a.physical_counts[i] = -1;
   if (threadIdx.x == 0) {
-    agent_store(sync + 0, 0);
-    agent_store(sync + 1, 0);
+    const int n_feasible = (int)((unsigned)summary >> 24);
+    if (!failed && n_feasible > 0)
+      atomicAdd(a.avail, n_feasible);
+    agent_store(a.sync + kLeftAt, 0);
+#ifdef LPLB_PHASE_CLOCKS
+    if (a.solve.clocks)
+      a.solve.clocks[113] = wall_clock64();
+#endif
   }
 }
 
-// LDS of a slice workgroup.
-static size_t plan_lds_bytes(int n_logical, int n_waves) {
-  const size_t groups = (size_t)n_waves * kWave >= (size_t)n_logical ? (size_t)n_waves * kWave / n_logical : 1;
-  return (size_t)n_logical * (sizeof(ExpertEntry) + 4 + 4 + (size_t)n_waves * (sizeof(WaveSlot) + 4) + groups * 8);
+// LDS of a slice workgroup: route and histogram per logical expert, a ranking record per
+// (wave, replicated set), the constants of the sets.
+static size_t plan_lds_bytes(int n_logical, int n_rep, int n_waves, int k) {
+  return (size_t)(n_rep + 1) * sizeof(RepEntry) + (size_t)n_waves * (n_rep + 1) * rank_record_bytes_single(k) +
+         (size_t)(n_logical + 1) * sizeof(Route) + (size_t)n_logical * sizeof(int32_t) +
+         (size_t)(3 + n_waves) * n_rep * sizeof(int32_t) + 16;
 }
 
-// Debug builds: stamps of the first and the last slice workgroup and of the LP's.
+// Debug builds: stamps of the first and the last slice workgroup and of the first LP workgroup.
 #define LPLB_PLAN_STAMP(k)                                                                     \
   LPLB_STAMP_AT(a.solve.clocks == nullptr ? nullptr                                            \
-                : blockIdx.x == 0 ? a.solve.clocks + 64                                        \
-                : blockIdx.x == a.n_slices - 1 ? a.solve.clocks + 80                           \
-                : blockIdx.x == a.n_slices ? a.solve.clocks + 96 : nullptr, k)
+                : blockIdx.x == a.n_lp_workgroups ? a.solve.clocks + 64                        \
+                : blockIdx.x == gridDim.x - 1 ? a.solve.clocks + 80                            \
+                : blockIdx.x == 0 ? a.solve.clocks + 96 : nullptr, k)
 
 // K: 64-index chunks per wave.  WAVES: waves per workgroup.
+// Registers: with LP shapes that fit 128 VGPRs the kernel as a whole is held to 128 (four
+// waves per SIMD: one 16-wave or two 8-wave workgroups per CU), which is what lets the 257
+// workgroups of a [262144 x 8] batch be resident together.
 template <int GM, int DM, bool EXACT, int K, int WAVES>
-__global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
+__global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) void plan_in_one_launch(PlanArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __shared__ int rep_of_edge_all[WAVES * kWave];
-  const int nl = a.sh.n_logical;
+  __shared__ int rep_of_edge_all[kLpsPerWorkgroup * kWave];
+  __shared__ int flags[4];   // [0] the exchange of counts worked, [1] some share will not come,
+                             // [2] a wait of this workgroup ran out, [3] feasible LPs of this workgroup
+  const int nl = a.sh.n_logical, R = a.n_rep;
   const int tid = threadIdx.x;
   constexpr int nt = WAVES * kWave;
-  const int lane = tid % kWave, wave = tid / kWave;
-  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // the same, but known to be wave-uniform
+  const int lane = tid % kWave;
+  const int wave_s = __builtin_amdgcn_readfirstlane(tid / kWave);   // wave-uniform
   const int pid = blockIdx.x;
-  const int n_workgroups = a.n_slices + a.n_lp_workgroups;
   const int n_shares = a.sh.n_ranks * a.sh.D;
-  const int n_groups = nt >= nl ? nt / nl : 1;   // threads per expert when rows are added up
+  unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
+  unsigned long long *totals_acc = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt);   // [n_copies][nl]
+  // The batch's tokens of expert e and the number of slices that have contributed: the copies
+  // added up (all loads in flight together); complete once every slice has arrived.
+  auto batch_totals = [&](int e, int32_t &tokens, int32_t &slices) {
+    unsigned long long v[kTotalCopies];
+#pragma unroll
+    for (int k = 0; k < kTotalCopies; ++k)
+      v[k] = totals_acc[(k & (a.n_copies - 1)) * nl + e];
+    unsigned long long sum = 0;
+#pragma unroll
+    for (int k = 0; k < kTotalCopies; ++k)
+      sum += k < a.n_copies ? v[k] : 0ull;
+    tokens = (int32_t)(sum >> 32);
+    slices = (int32_t)(uint32_t)sum;
+  };
 
-  if (pid >= a.n_slices) {
+  if (pid < a.n_lp_workgroups) {
     // ------------------------------------------------------------ the LPs
     SolveArgs sa = a.solve;
-    const int first_lp = (pid - a.n_slices) * kLpsPerWorkgroup;          // of this workgroup
+    const int first_lp = pid * kLpsPerWorkgroup;          // of this workgroup
     const int n_lps = min(kLpsPerWorkgroup, sa.n_units - first_lp);
     LPLB_PLAN_STAMP(0);
     // Own-histogram mode: the LP waves start at once (their table loads do not need
@@ -185,246 +217,387 @@ __global__ __launch_bounds__(WAVES *kWave) void plan_in_one_launch(PlanArgs a) {
     // slices, fetches the totals the slices have added up in memory and hands them over.
     __shared__ int counts_ready;
     float *staged = reinterpret_cast<float *>(smem_raw);
+    if (tid == 0) {
+      counts_ready = 0;
+      flags[2] = 0;
+      flags[3] = 0;
+    }
+    __syncthreads();
     if (a.local_counts) {
-      if (tid == 0)
-        counts_ready = 0;
-      __syncthreads();
       sa.counts_ready = &counts_ready;
-      if (wave == n_lps) {
-        // Poll the totals until every expert's word says that all slices have added
-        // theirs (plain loads after an acquire fence: they can be batched).
-        const unsigned long long *words = reinterpret_cast<const unsigned long long *>(a.sync + kTotalsAt);
-        for (int polls = 0;; ++polls) {
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      if (wave_s == n_lps) {
+        // Poll the batch's totals until every expert's words say that all slices have
+        // added theirs (plain loads after an acquire: they can be batched).
+        bool complete = false;
+        for (int polls = 0; polls < a.max_polls && !complete; ++polls) {
+          see_other_workgroups();
           bool all_in = true;
-          for (int e0 = lane; e0 < nl; e0 += 8 * kWave) {
-            unsigned long long t[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-              t[k] = words[min(e0 + k * kWave, nl - 1)];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-              all_in = all_in && (uint32_t)t[k] == (uint32_t)a.n_slices;
-              if (e0 + k * kWave < nl)
-                staged[e0 + k * kWave] = (float)(uint32_t)(t[k] >> 32);
-            }
+          for (int e = lane; e < nl; e += kWave) {
+            int32_t tokens, slices;
+            batch_totals(e, tokens, slices);
+            all_in = all_in && slices == a.expected_slices;
+            staged[e] = (float)tokens;
           }
-          if (__all(all_in))
-            break;
-          if (polls >= kMaxPolls) {
-            if (lane == 0)
-              __hip_atomic_fetch_add(a.sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-          __builtin_amdgcn_s_sleep(2);
+          complete = __all(all_in);
+          if (!complete)
+            __builtin_amdgcn_s_sleep(2);
         }
-        if (pid == a.n_slices)
-          for (int e = lane; e < nl; e += kWave)   // this GPU's totals, for the caller
-            a.totals[e] = (int32_t)staged[e];
+        if (!complete && lane == 0) {
+          give_up(a);
+          flags[2] = 1;
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
-          __hip_atomic_store(&counts_ready, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          __hip_atomic_store(&counts_ready, complete ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
     }
     LPLB_PLAN_STAMP(1);
-    if (wave < n_lps) {
+    if (wave_s < n_lps) {
       // (own-histogram mode: every LP of the batch reads the one staged copy)
-      float *mine = a.local_counts ? staged : staged + (size_t)wave * sa.staged_stride;
-      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, first_lp + wave, mine, rep_of_edge_all + wave * kWave);
-      if (lane == 0 && n_ok > 0)
-        atomicAdd(sa.avail, n_ok);
+      float *mine = a.local_counts ? staged : staged + (size_t)wave_s * sa.staged_stride;
+      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, first_lp + wave_s, mine, rep_of_edge_all + wave_s * kWave);
+      if (n_ok < 0) {
+        // no counts, no solution: tell the slices not to wait for this LP's shares
+        const int n_edges = sa.G * sa.D;
+        for (int j = lane; j < n_edges; j += kWave)
+          agent_store(shares + (int64_t)(first_lp + wave_s) * n_edges + j, 2ull << 32);
+      } else if (lane == 0 && n_ok > 0) {
+        atomicAdd(&flags[3], n_ok);
+      }
     }
     LPLB_PLAN_STAMP(2);
-    leave(a.sync, n_workgroups, n_shares, a.local_counts ? nl : 0);
+    leave(a, n_shares, &flags[2], &flags[3]);
     return;
   }
 
   // --------------------------------------------------------------- a slice
-  ExpertEntry *table = reinterpret_cast<ExpertEntry *>(smem_raw);              // [nl]
-  WaveSlot *slots = reinterpret_cast<WaveSlot *>(table + nl);                 // [WAVES][nl]
-  int32_t *replica = reinterpret_cast<int32_t *>(slots + (size_t)WAVES * nl); // [nl]
-  int32_t *start = replica + nl;                                              // [nl]
-  int32_t *counts = start + nl;                                               // [WAVES][nl]
-  int32_t *partial = counts + (size_t)WAVES * nl;                             // [2][n_groups][nl]
-  WaveSlot *mine = slots + (size_t)wave * nl;
+  constexpr int kRec = rank_record_bytes_single(K);
+  const int slice = pid - a.n_lp_workgroups;
+  RepEntry *reps = reinterpret_cast<RepEntry *>(smem_raw);                          // [R + 1]
+  unsigned char *records = smem_raw + (size_t)(R + 1) * sizeof(RepEntry);          // [WAVES][R + 1][kRec]
+  const int wave_stride = (R + 1) * kRec;
+  Route *route = reinterpret_cast<Route *>(records + (size_t)WAVES * wave_stride);  // [nl + 1]
+  int32_t *hist = reinterpret_cast<int32_t *>(route + nl + 1);                      // [nl]
+  int32_t *set_expert = hist + nl;                                                  // [R]
+  int32_t *before = set_expert + R;                                                 // [R] tokens of the set before this slice
+  int32_t *total = before + R;                                                      // [R] ... in the whole batch
+  int32_t *wave_total = total + R;                                                  // [WAVES][R] ... in each wave's chunks
+  unsigned char *my_records = records + (size_t)wave_s * wave_stride;
   const unsigned long long my_bit = 1ull << lane;
-  const int64_t begin = slice_begin(a.n, a.per, pid);
-  const int64_t end = slice_begin(a.n, a.per, pid + 1);
-
+  const int64_t begin = slice_begin(a.n, a.per, slice);
+  const int64_t end = slice_begin(a.n, a.per, slice + 1);
+  const int cd = a.sh.C * a.sh.D;
   LPLB_PLAN_STAMP(0);
-  // Small table reads that depend on nothing go out first; they are used much later.
-  const int cd = a.sh.C * a.sh.D, n_sets = a.sh.n_ranks * cd;
-  const int le_of_tid = tid < nl ? a.phy2log[(tid / a.sh.L) * a.sh.P + (tid % a.sh.L)] : -1;
-  // first (usually only) replicated expert set of this thread
-  const bool set0 = tid < n_sets;
-  const int rank0 = set0 ? tid / cd : 0, local0 = set0 ? tid % cd : 0;
-  const int rle0 = set0 ? a.phy2log[rank0 * a.sh.P + local0] : -1;
-  const int host0 = set0 ? a.o2r[(rank0 % a.sh.G) * a.sh.D + local0 % a.sh.D] : 0;
-  int32_t ev[K];   // expert ids, -1 for masked / out-of-range / past the end
+
+  // ---- small table reads first (they need no counts), then the index loads; all of
+  // them unconditional loads from clamped addresses, so that nothing waits here ----
+  auto slot_of = [&](int e) { return e + (int)fast_div((uint32_t)e, a.magic_L) * (a.sh.P - a.sh.L); };
+  struct SetOf {
+    int ep_rank, place, d, group_rank;
+  };
+  auto set_of = [&](int i) {
+    SetOf s;
+    s.ep_rank = (int)fast_div((uint32_t)i, a.magic_cd);
+    s.place = i - s.ep_rank * cd;
+    s.d = s.place - (int)fast_div((uint32_t)s.place, a.magic_D) * a.sh.D;
+    s.group_rank = s.ep_rank - (int)fast_div((uint32_t)s.ep_rank, a.magic_G) * a.sh.G;
+    return s;
+  };
+  const int e0 = min(tid, nl - 1);
+  const int slot0 = slot_of(e0);
+  const int le0 = a.phy2log[slot0];
+  const bool set0 = tid < R;
+  const SetOf s0 = set_of(set0 ? tid : 0);
+  const int rle0 = a.phy2log[s0.ep_rank * a.sh.P + s0.place];
+  const int host0 = a.o2r[s0.group_rank * a.sh.D + s0.d];
+  const int64_t w0 = begin + (int64_t)wave_s * (K * kWave);   // first index of this wave's K chunks (uniform)
+  const bool whole = w0 + K * kWave <= end;
+  int64_t raw[K];
+  {
+    const int64_t *src = a.idx + w0 + lane;
+    if (whole) {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        raw[c] = __builtin_nontemporal_load(src + c * kWave);
+    } else {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        raw[c] = w0 + c * kWave + lane < end ? __builtin_nontemporal_load(src + c * kWave) : -1;
+    }
+  }
+
+  // ---- tables that need phy2log only: where an expert's tokens go when nothing is
+  // redirected, and which replicated set (if any) it belongs to; minilp.cu:466-496 ----
+  for (int e = tid; e <= nl; e += nt)
+    route[e] = Route{-1, R};
+  for (int e = tid; e < nl; e += nt)
+    hist[e] = 0;
+  {
+    const i32x4 zero{0, 0, 0, 0};
+    i32x4 *z = reinterpret_cast<i32x4 *>(records);
+    for (int i = tid; i < WAVES * wave_stride / 16; i += nt)
+      z[i] = zero;
+  }
+  for (int q = tid; q < R; q += nt) {
+    before[q] = 0;
+    total[q] = 0;
+  }
+  if (tid == 0) {
+    reps[R] = RepEntry{1, 0xffffffffu, INT32_MAX, -1};   // "no replica": every token stays
+    flags[0] = 0;
+    flags[1] = 0;
+    flags[3] = 0;
+  }
+  __syncthreads();
+  if (tid < nl && le0 >= 0 && le0 < nl)
+    route[le0].original = slot0;
+  for (int e = tid + nt; e < nl; e += nt) {
+    const int s = slot_of(e), le = a.phy2log[s];
+    if (le >= 0 && le < nl)
+      route[le].original = s;
+  }
+  // A set's key is R - 1 - i, so that of two sets that name the same expert the later one
+  // wins (as a sequential pass over the sets would have it) with an atomic min.
+  auto enter_set = [&](int i, const SetOf &s, int le, int host) {
+    const bool ok = le >= 0 && le < nl;
+    if (ok)
+      atomicMin(&route[le].rep, R - 1 - i);
+    reps[R - 1 - i] = RepEntry{0, 0u, 0, ((s.ep_rank - s.group_rank) + host + 1) * a.sh.P - cd + s.place};
+    set_expert[R - 1 - i] = ok ? le : -1;
+  };
+  if (set0)
+    enter_set(tid, s0, rle0, host0);
+  for (int i = tid + nt; i < R; i += nt) {
+    const SetOf s = set_of(i);
+    enter_set(i, s, a.phy2log[s.ep_rank * a.sh.P + s.place], a.o2r[s.group_rank * a.sh.D + s.d]);
+  }
+  __syncthreads();
+
+  // ---- the tokens: histogram of the slice, bitmaps of the replicated sets per chunk ----
+  // Between the phases a token is kept as its expert id only, two ids per register (the
+  // route is looked up again where it is needed): the waits below are long and registers
+  // are what bounds how many workgroups are resident.
+  uint32_t packed[(K + 1) / 2];
+  auto expert_of_chunk = [&](int c) { return (int)((packed[c / 2] >> (16 * (c % 2))) & 0xffffu); };
+  auto slot_of_chunk = [&](int set, int c) {
+    return reinterpret_cast<ChunkSlot *>(my_records + __umul24((uint32_t)set, (uint32_t)kRec)) + c;
+  };
 #pragma unroll
   for (int c = 0; c < K; ++c) {
-    const int64_t i = begin + ((int64_t)wave * K + c) * kWave + lane;
-    const int64_t v = i < end ? __builtin_nontemporal_load(a.idx + i) : -1;
-    ev[c] = (v >= 0 && v < nl) ? (int32_t)v : -1;
-  }
-  for (int i = tid; i < WAVES * nl; i += nt) {
-    slots[i] = WaveSlot{0, 0, 0ull};
-    counts[i] = 0;
+    const bool valid = (uint64_t)raw[c] < (uint64_t)nl;   // -1, other negatives and too large ids fail
+    const int e = valid ? (int)raw[c] : nl;
+    packed[c / 2] = (c % 2) ? packed[c / 2] | ((uint32_t)e << 16) : (uint32_t)e;
+    const int set = route[e].rep;
+    // a token of a replicated set is counted through the set's bitmaps (the sets hold the hot
+    // experts, whose tokens would queue up at one histogram counter), any other one here
+    if (set < R)
+      atomicOr(reinterpret_cast<unsigned long long *>(slot_of_chunk(set, c)), my_bit);
+    else if (valid)
+      atomicAdd(&hist[e], 1);
   }
   __syncthreads();
-  // tokens per expert in this wave's chunks
-#pragma unroll
-  for (int c = 0; c < K; ++c)
-    if (ev[c] >= 0)
-      atomicAdd(&counts[(size_t)wave * nl + ev[c]], 1);
+  // ---- inside the wave: tokens of each set in the chunks before each chunk (lane = (set,
+  // chunk), chunk fastest), and in all of the wave's chunks ----
+  if (R > 0) {
+    const int c = lane % K;
+    for (int p0 = 0; p0 < R * K; p0 += kWave) {
+      const bool live = p0 + lane < R * K;
+      const int q = live ? (p0 + lane) / K : R;   // lanes past the end read the stand-in record (zeros)
+      ChunkSlot *mine = reinterpret_cast<ChunkSlot *>(my_records + __umul24((uint32_t)q, (uint32_t)kRec)) + c;
+      const int own = __popcll(*reinterpret_cast<const unsigned long long *>(mine));
+      const int in_my_wave = group_sum<K>(own);
+      const int in_earlier_chunks = group_exclusive_scan<K>(own, c);
+      if (live) {
+        mine->start = in_earlier_chunks;
+        if (c == 0)
+          wave_total[wave_s * R + q] = in_my_wave;
+      }
+    }
+  }
   __syncthreads();
-  // this slice's histogram row, for every workgroup to read
-  for (int e = tid; e < nl; e += nt) {
-    int32_t h = 0;
-#pragma unroll
+  for (int q = tid; q < R; q += nt) {   // the sets' tokens in this slice, into the histogram
+    int32_t n = 0;
     for (int w = 0; w < WAVES; ++w)
-      h += counts[(size_t)w * nl + e];
-    agent_store(a.rows + (int64_t)pid * nl + e, h);
-    if (a.local_counts)
-      __hip_atomic_fetch_add(reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + e,
-                             ((unsigned long long)(uint32_t)h << 32) | 1ull, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+      n += wave_total[w * R + q];
+    const int le = set_expert[q];
+    if (le >= 0 && route[le].rep == q)   // (of two sets that name the same expert only one has the tokens)
+      hist[le] = n;
   }
-  __builtin_amdgcn_s_waitcnt(0);   // the row has left this CU
+  __syncthreads();
+  // ---- this slice's counts, for every workgroup: the histogram goes into the batch's
+  // totals, the counts of the replicated sets into this slice's row ----
+  for (int e = tid; e < nl; e += nt) {
+    const int32_t mine = hist[e];
+    if (a.local_counts || mine != 0)   // (only the LP's poller looks at the number of contributions)
+      agent_add(totals_acc + (slice & (a.n_copies - 1)) * nl + e, ((unsigned long long)(uint32_t)mine << 32) | 1ull);
+  }
+  for (int q = tid; q < R; q += nt) {
+    const int le = set_expert[q];
+    agent_store(a.rows + (((int64_t)slice) << a.row_shift) + q, le >= 0 ? hist[le] : 0);
+  }
+  stores_have_landed();
   __syncthreads();
   LPLB_PLAN_STAMP(1);
-  if (tid == 0) {
-    __hip_atomic_fetch_add(a.sync + 0, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    wait_for(a.sync, 0, a.n_slices);
+  if (wave_s == 0) {
+    if (lane == 0)
+      announce_arrival(a.sync + kArrivedAt, slice);
+    const bool arrived = wait_for_arrivals(a.sync + kArrivedAt, a.expected_slices, a.max_polls);
+    if (lane == 0) {
+      if (!arrived)
+        give_up(a);
+      flags[0] = arrived;
+    }
   }
   __syncthreads();
   LPLB_PLAN_STAMP(2);
-  // add up the rows: tokens per expert in the whole batch and before this slice
-  {
-    const int g = nt >= nl ? tid / nl : 0;
-    if (g < n_groups)
-      for (int e = nt >= nl ? tid % nl : tid; e < nl; e += nt >= nl ? nl : nt) {
-        int32_t t, before;
-        add_up_rows(a.rows, a.n_slices, nl, e, g, n_groups, pid, t, before);
-        partial[(size_t)g * nl + e] = t;
-        partial[(size_t)(n_groups + g) * nl + e] = before;
-      }
-  }
-  __syncthreads();
-  LPLB_PLAN_STAMP(6);
-  for (int e = tid; e < nl; e += nt) {
-    int32_t t = 0, before = 0;
-    for (int g = 0; g < n_groups; ++g) {
-      t += partial[(size_t)g * nl + e];
-      before += partial[(size_t)(n_groups + g) * nl + e];
-    }
-    init_entry(table, replica, start, e, t, before);
-    if (pid == 0 && !a.local_counts)
-      a.totals[e] = t;
-  }
-  __syncthreads();
-  if (tid < nl)
-    set_original(table, a.sh, tid, le_of_tid);
-  for (int e = tid + nt; e < nl; e += nt)
-    set_original(table, a.sh, e, a.phy2log[(e / a.sh.L) * a.sh.P + (e % a.sh.L)]);
-  LPLB_PLAN_STAMP(7);
-  // each wave's starting ordinals: tokens before this slice + those of the waves before
-  // it; specialised by the (wave-uniform) number of those, so that the loop is
-  // straight-line with exactly that many reads
-  static_for<WAVES>([&](auto wc) {
-    constexpr int kEarlier = decltype(wc)::value;
-    if (wave_s != kEarlier)
-      return;
-    for (int e = lane; e < nl; e += kWave) {
-      int32_t before[kEarlier + 1];
-#pragma unroll
-      for (int w = 0; w < kEarlier; ++w)
-        before[w] = counts[(size_t)w * nl + e];
-      int32_t run = start[e];
-#pragma unroll
-      for (int w = 0; w < kEarlier; ++w)
-        run += before[w];
-      mine[e].next = run;
-    }
-  });
-  // The LP's shares decide how many tokens stay on the original, and nothing else:
-  // replica slots, ordinals and hashes are worked out while the LP is still running,
-  // so that one multiplication and one comparison per token are left for afterwards.
-  LPLB_PLAN_STAMP(3);
-  const unsigned long long *shares = reinterpret_cast<const unsigned long long *>(a.sync + kSharesAt);
-  int le0 = -1;
-  int32_t total0 = 0;
-  if (set0) {
-    set_replica_slot(replica, a.sh, rank0, local0, rle0, host0);
-    if (rle0 >= 0 && rle0 < nl) {
-      le0 = rle0;
-      total0 = table[le0].total;
-    }
-  }
-  for (int i = tid + nt; i < n_sets; i += nt) {
-    const int ep_rank = i / cd, local = i % cd;
-    set_replica_slot(replica, a.sh, ep_rank, local, a.phy2log[ep_rank * a.sh.P + local],
-                     a.o2r[(ep_rank % a.sh.G) * a.sh.D + local % a.sh.D]);
-  }
-  __builtin_amdgcn_wave_barrier();   // the wave's starting ordinals above are read by other lanes below
+  bool ok = flags[0] != 0;   // (the same in every thread)
   int32_t h[K];
+  if (ok) {
+    // (wave 0's wait ended with the acquire that lets the plain loads below see the other
+    // workgroups' rows: one invalidate per workgroup, not one per wave)
+    // ---- tokens of each replicated set before this slice and in the whole batch: a thread
+    // takes one set of every (threads / row length)-th slice, loads in batches ----
+    {
+      const int row_len = 1 << a.row_shift;
+      const int q_lanes = min(row_len, nt), p_lanes = nt / q_lanes;   // powers of two
+      const int p_first = tid / q_lanes;
+      constexpr int kInFlight = 8;
+      for (int q = tid % q_lanes; q < R; q += q_lanes) {
+        int32_t t_sum = 0, b_sum = 0;
+        for (int p0 = p_first; p0 < a.n_slices; p0 += kInFlight * p_lanes) {
+          int32_t v[kInFlight];
 #pragma unroll
-  for (int c = 0; c < K; ++c) {
-    ExpertEntry unused;
-    h[c] = hash_of_token<false>(ev[c], mine, table, my_bit, unused);
-    __builtin_amdgcn_wave_barrier();
-  }
-  // Every thread that needs a share polls it itself: value and "valid" arrive in the
-  // same 8-byte word.
-  auto share_of = [&](int ep_rank, int d) {
-    unsigned long long word = 0;
-    int polls = 0;
-    while ((word = __hip_atomic_load(shares + ep_rank * a.sh.D + d, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT)) == 0 && ++polls < kMaxPolls)
-      __builtin_amdgcn_s_sleep(2);
-    if (polls >= kMaxPolls)
-      __hip_atomic_fetch_add(a.sync + 3, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return __builtin_bit_cast(float, (uint32_t)word);
-  };
-  if (set0) {
-    const float share = share_of(rank0, local0 % a.sh.D);
-    if (le0 >= 0)
-      table[le0].expected = expected_on_original(share, total0);
-  }
-  for (int i = tid + nt; i < n_sets; i += nt) {
-    const int ep_rank = i / cd, local = i % cd;
-    const float share = share_of(ep_rank, local % a.sh.D);
-    const int le = a.phy2log[ep_rank * a.sh.P + local];
-    if (le >= 0 && le < nl)
-      table[le].expected = expected_on_original(share, table[le].total);
-  }
-  __syncthreads();
+          for (int k = 0; k < kInFlight; ++k)
+            v[k] = a.rows[(((int64_t)min(p0 + k * p_lanes, a.n_slices - 1)) << a.row_shift) + q];
 #pragma unroll
-  for (int c = 0; c < K; ++c) {
-    int64_t o = -1;
-    if (ev[c] >= 0) {
-      const ExpertEntry x = table[ev[c]];
-      o = h[c] >= x.expected ? replica[ev[c]] : x.original;
+          for (int k = 0; k < kInFlight; ++k) {
+            const int p = p0 + k * p_lanes;
+            t_sum += p < a.n_slices ? v[k] : 0;
+            b_sum += p < slice ? v[k] : 0;
+          }
+        }
+        atomicAdd(&total[q], t_sum);
+        atomicAdd(&before[q], b_sum);
+      }
     }
-    const int64_t i = begin + ((int64_t)wave * K + c) * kWave + lane;
-    if (i < end)
-      __builtin_nontemporal_store(o, a.out + i);
+    if (slice == 0)   // this GPU's tokens per expert, for the caller (and for the counts below)
+      for (int e = tid; e < nl; e += nt) {
+        int32_t tokens, slices;
+        batch_totals(e, tokens, slices);
+        a.totals[e] = tokens;
+        hist[e] = tokens;
+      }
+    __syncthreads();
+    LPLB_PLAN_STAMP(3);
+    for (int q = tid; q < R; q += nt) {
+      const int32_t t = total[q];
+      reps[q].total = t;
+      reps[q].magic = t >= 1 ? 0xffffffffu / (uint32_t)t : 0u;
+    }
+    // ---- ordinal of the first token of every (wave, set, chunk): what is there already
+    // (tokens in the wave's earlier chunks) plus the tokens before this slice and in the
+    // waves before this one ----
+    if (R > 0) {
+      const int c = lane % K;
+      for (int p0 = 0; p0 < R * K; p0 += kWave) {
+        const bool live = p0 + lane < R * K;
+        const int q = live ? (p0 + lane) / K : 0;
+        int32_t base = before[q];
+        for (int v0 = 0; v0 < wave_s; v0 += 4) {
+          int32_t t[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            t[u] = wave_total[min(v0 + u, wave_s) * R + q];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            base += v0 + u < wave_s ? t[u] : 0;
+        }
+        if (live)
+          atomicAdd(&(reinterpret_cast<ChunkSlot *>(my_records + __umul24((uint32_t)q, (uint32_t)kRec)) + c)->start, base);
+      }
+    }
+    __syncthreads();
+    LPLB_PLAN_STAMP(4);
+    // ---- ordinals and hashes of the tokens, while the LP is still running ----
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const int set = route[expert_of_chunk(c)].rep;
+      const i32x4 s = *reinterpret_cast<const i32x4 *>(slot_of_chunk(set, c));   // bits_lo, bits_hi, start
+      const i32x4 x = *reinterpret_cast<const i32x4 *>(&reps[set]);              // total, magic, -, -
+      const int32_t k =
+          __builtin_amdgcn_mbcnt_hi((uint32_t)s.y, __builtin_amdgcn_mbcnt_lo((uint32_t)s.x, (uint32_t)s.z));
+      h[c] = ordinal_hash<false>(k, x.x, (uint32_t)x.y);
+    }
+    // ---- the LP's shares: every set's thread polls its own; value and tag arrive in
+    // the same 8-byte word ----
+    for (int i = tid; i < R; i += nt) {
+      const SetOf s = set_of(i);
+      unsigned long long word = 0;
+      int polls = 0;
+      while ((word = agent_load(shares + s.ep_rank * a.sh.D + s.d)) == 0 && ++polls < a.max_polls)
+        __builtin_amdgcn_s_sleep(2);
+      if ((uint32_t)(word >> 32) == 1u) {
+        reps[R - 1 - i].expected = expected_on_original(__builtin_bit_cast(float, (uint32_t)word), total[R - 1 - i]);
+      } else {
+        if (word == 0)
+          give_up(a);
+        flags[1] = 1;
+      }
+    }
+    __syncthreads();
+    LPLB_PLAN_STAMP(5);
+    ok = flags[1] == 0;
   }
-  if (pid == 0 && a.physical_counts)
-    emit_physical_counts(table, replica, a.sh, a.phy2log, a.physical_counts, tid, nt);
-  LPLB_PLAN_STAMP(5);
-  leave(a.sync, n_workgroups, n_shares, a.local_counts ? nl : 0);
-}
-
-template <int GM, int DM, bool EXACT, int K, int WAVES>
-static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t s) {
-  if (lds > 64 * 1024) {
-    const hipError_t err = allow_dynamic_lds(&plan_in_one_launch<GM, DM, EXACT, K, WAVES>, kPlanLdsLimit);
-    if (err != hipSuccess)
-      return err;
+  // Tokens per physical expert (= bincount of the output) from the first slice's tables.
+  if (slice == 0 && a.physical_counts && ok) {
+    for (int i = tid; i < a.sh.n_ranks * a.sh.P; i += nt) {
+      const int le = a.phy2log[i];
+      int32_t v = 0;
+      if (le >= 0 && le < nl) {
+        const Route rt = route[le];
+        if (rt.rep >= R) {
+          v = rt.original == i ? hist[le] : 0;   // (slice 0 keeps the batch's totals there)
+        } else {
+          const RepEntry x = reps[rt.rep];
+          const int32_t kept = kept_on_original(x.total, x.expected);
+          v = rt.original == i ? kept : (x.replica == i ? x.total - kept : 0);
+        }
+      }
+      a.physical_counts[i] = v;
+    }
+    stores_have_landed();   // (a launch that gave up overwrites them from the last workgroup to leave)
   }
-  launch(plan_in_one_launch<GM, DM, EXACT, K, WAVES>, dim3(a.n_slices + a.n_lp_workgroups), dim3(WAVES * kWave), lds, s, a);
-  return hipGetLastError();
+  // This workgroup needs nothing from the others any more: it counts as gone now, so that the
+  // counters are cleared while the outputs are still being stored, not after them.
+  LPLB_PLAN_STAMP(6);
+  if (tid == 0)
+    flags[2] = !ok;
+  leave(a, n_shares, &flags[2], &flags[3]);
+  // ---- choose and store; if a wait ran out, every token goes to its original slot ----
+  {
+    int64_t *dst = a.out + w0 + lane;
+    int32_t o[K];
+#pragma unroll
+    for (int c = 0; c < K; ++c) {
+      const Route rt = route[expert_of_chunk(c)];
+      o[c] = rt.original;
+      if (ok) {
+        const RepEntry x = reps[rt.rep];
+        o[c] = h[c] >= x.expected ? x.replica : rt.original;
+      }
+    }
+    if (whole) {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        __builtin_nontemporal_store((int64_t)o[c], dst + c * kWave);
+    } else {
+#pragma unroll
+      for (int c = 0; c < K; ++c)
+        if (w0 + c * kWave + lane < end)
+          __builtin_nontemporal_store((int64_t)o[c], dst + c * kWave);
+    }
+  }
+  LPLB_PLAN_STAMP(7);
 }
 
 // LP shapes the one-launch plan is built for, in the order they are tried, and the
@@ -432,6 +605,7 @@ static hipError_t launch_plan_variant(const PlanArgs &a, size_t lds, hipStream_t
 // 256 at 8.
 constexpr int kPlanShapes[][2] = {{8, 1}, {8, 2}, {8, 4}, {16, 1}, {16, 2}, {32, 1}, {32, 2}};
 constexpr int plan_waves(int gm, int dm) { return (gm * dm <= 16 && gm <= 16) ? 16 : 8; }
+constexpr int plan_max_chunks(int waves) { return waves == 16 ? 8 : 16; }   // longest slice: 8192 indices
 static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
   for (const auto &shape : kPlanShapes)
     if (G <= shape[0] && D <= shape[1]) {
@@ -442,58 +616,205 @@ static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
   return false;
 }
 
-template <int GM, int DM, bool EXACT, int W> static hipError_t launch_plan_shape(PlanArgs &a, hipStream_t s) {
-  const int64_t chunks = (a.per + kWave - 1) / kWave;
-  const int k = (int)((chunks + W - 1) / W);
-  const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, W);
-  const size_t lds_lp = (size_t)min(a.solve.n_units, kLpsPerWorkgroup) * a.solve.n_experts * sizeof(float);
-  a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
-  if (a.local_counts && a.solve.staged_stride == 0)   // the LP takes its counts from LDS in that mode
-    return hipErrorInvalidValue;
-  if (k <= 1)
-    return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s);
-  if (k <= 2)
-    return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds_slices, s);
-  if (k <= 4)
-    return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s);
-  return launch_plan_variant<GM, DM, EXACT, 8, W>(a, lds_slices, s);
-}
+// ---- host side: which launches may run as one kernel ----
+// Per device: the counters' address and, per slot, which stream owns it and what its
+// launches cost.  A slot belongs to one stream at a time (launches that share a slot must
+// not overlap, which stream order guarantees); a slot whose stream has no work pending may
+// pass to another stream.  A slot with a launch captured into a graph stays with its stream
+// for good and counts as executing for good: a replay may come at any time and the host
+// does not see it.
+struct PlanSlot {
+  hipStream_t stream = nullptr;
+  float cost = 0.0f;            // share of the GPU's resident workgroups its launches take
+  bool used = false, captured = false;
+  bool maybe_executing = false; // a launch was enqueued and the stream has not been seen idle since
+};
+struct PlanDevice {
+  int *sync = nullptr;
+  int n_cus = 0;
+  PlanSlot slots[kSyncSlots];
+};
+static std::mutex g_plan_guard;
+static PlanDevice g_plan_devices[64];
+// Up to this share of the GPU's resident workgroups may belong to plans that wait for
+// their own workgroups; the rest stays free for their stragglers and for other kernels.
+constexpr float kResidencyBudget = 0.80f;
 
-// The block of counters a stream uses: the first kSyncSlots streams that run a plan
-// each get their own, -1 for any further one (which then runs the chain).
-static int sync_slot_of(hipStream_t s) {
-  static std::mutex guard;
-  static hipStream_t owner[kSyncSlots];
-  static int used = 0;
-  std::lock_guard<std::mutex> lock(guard);
-  for (int i = 0; i < used; ++i)
-    if (owner[i] == s)
-      return i;
-  if (used == kSyncSlots)
-    return -1;
-  owner[used] = s;
-  return used++;
-}
-
-// Per-device address of the counters and CU count, looked up once (threads that race
-// for the first look-up store the same values).
-static int plan_device_state(int **sync, int *n_cus) {
-  static std::atomic<int *> sync_of[64];
+// Looks the per-device state up.
+static int plan_device(PlanDevice **out) {
   int dev = -1;
   LPLB_HIP_TRY(hipGetDevice(&dev));
   LPLB_REQUIRE(dev >= 0 && dev < 64, LPLB_EUNSUPPORTED, "plan: device ordinal %d", dev);
-  int *p = sync_of[dev].load(std::memory_order_acquire);
-  if (!p) {
-    LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(g_plan_sync)));
-    sync_of[dev].store(p, std::memory_order_release);
+  PlanDevice &d = g_plan_devices[dev];
+  static std::mutex first_use;
+  std::lock_guard<std::mutex> lock(first_use);
+  if (!d.sync) {
+    int *sync = nullptr;
+    LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&sync), HIP_SYMBOL(g_plan_sync)));
+    d.n_cus = current_device_cu_count();
+    LPLB_REQUIRE(d.n_cus > 0, LPLB_EHIP, "plan: cannot read the CU count of device %d", dev);
+    d.sync = sync;
   }
-  *sync = p;
-  *n_cus = current_device_cu_count();
-  LPLB_REQUIRE(*n_cus > 0, LPLB_EHIP, "plan: cannot read the CU count of device %d", dev);
+  *out = &d;
   return LPLB_OK;
 }
 
-// Tries the one-launch plan.  *done = false: shape or size outside what it covers.
+// May a launch of this slot still be executing?  Asks the runtime whether the slot's stream
+// has work pending (any work: a stream busy with other kernels counts as executing, which
+// only errs towards the chain); never waits.
+// may_ask = false (the calling stream is being captured, and a stream query would break the
+// capture): what is not known to be idle counts as executing.
+static bool slot_is_executing(PlanDevice &d, int i, bool may_ask) {
+  PlanSlot &s = d.slots[i];
+  if (!s.used)
+    return false;
+  if (s.captured)
+    return true;
+  if (s.maybe_executing && may_ask && hipStreamQuery(s.stream) != hipErrorNotReady)
+    s.maybe_executing = false;   // idle (or the stream is gone)
+  return s.maybe_executing;
+}
+
+// Admission of one launch that takes `cost` of the GPU's resident workgroups on stream s.
+// Returns the slot, or -1: run the chain.
+static int admit_launch(PlanDevice &d, hipStream_t s, float cost, bool capturing) {
+  int slot = -1;
+  for (int i = 0; i < kSyncSlots && slot < 0; ++i)
+    if (d.slots[i].used && d.slots[i].stream == s)
+      slot = i;
+  for (int i = 0; i < kSyncSlots && slot < 0; ++i)
+    if (!d.slots[i].used)
+      slot = i;
+  for (int i = 0; i < kSyncSlots && slot < 0; ++i)
+    if (!slot_is_executing(d, i, !capturing))
+      slot = i;
+  if (slot < 0)
+    return -1;
+  float executing = 0.0f;
+  for (int i = 0; i < kSyncSlots; ++i)
+    if (i != slot && slot_is_executing(d, i, !capturing))
+      executing += d.slots[i].cost;
+  if (executing + cost > kResidencyBudget)
+    return -1;
+  PlanSlot &ps = d.slots[slot];
+  if (!ps.used || ps.stream != s) {
+    ps.stream = s;
+    ps.cost = 0.0f;
+    ps.used = true;
+    ps.captured = ps.maybe_executing = false;
+  }
+  ps.cost = ps.captured ? (cost > ps.cost ? cost : ps.cost) : cost;
+  ps.captured = ps.captured || capturing;
+  return slot;
+}
+
+// Workgroups of one kernel variant that fit a CU: bounded by the vector registers (512 per
+// SIMD lane, allocated in blocks of 8, at most 8 waves per SIMD) and by the LDS (160 KiB per
+// CU).  Worked out from the kernel's own attributes; the runtime's occupancy query changes
+// its answer once a kernel has been allowed more than 64 KiB of dynamic LDS.
+struct KernelFootprint {   // one per kernel variant (a static of launch_plan_variant)
+  std::atomic<int> regs{-1}, static_lds{0};
+};
+static int workgroups_per_cu(const void *kernel, KernelFootprint &known, int waves, size_t lds) {
+  int regs = known.regs.load(std::memory_order_acquire);
+  if (regs < 0) {
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, kernel) != hipSuccess || attr.numRegs <= 0)
+      return 0;
+    known.static_lds.store((int)attr.sharedSizeBytes, std::memory_order_relaxed);
+    regs = attr.numRegs;
+    known.regs.store(regs, std::memory_order_release);
+  }
+  const int per_wave = (regs + 7) / 8 * 8;
+  const int waves_per_simd = min(8, 512 / per_wave);
+  const int by_registers = waves_per_simd * 4 / waves;
+  const int by_lds = (int)((size_t)(160 * 1024) / (lds + (size_t)known.static_lds.load(std::memory_order_relaxed) + 256));
+  return min(by_registers, by_lds);
+}
+
+// Launches one variant if the whole grid fits the GPU beside the plans that are still
+// executing.  *done = false: it does not; nothing was enqueued.
+template <int GM, int DM, bool EXACT, int K, int WAVES>
+static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *done) {
+  auto kernel = plan_in_one_launch<GM, DM, EXACT, K, WAVES>;
+  if (lds > 64 * 1024)
+    LPLB_HIP_TRY(allow_dynamic_lds(kernel, kPlanLdsLimit));
+  PlanDevice *d = nullptr;
+  int rc = plan_device(&d);
+  if (rc != LPLB_OK)
+    return rc;
+  static KernelFootprint footprint;
+  const int fit = workgroups_per_cu(reinterpret_cast<const void *>(kernel), footprint, WAVES, lds);
+  const int n_workgroups = a.n_slices + a.n_lp_workgroups;
+#ifdef LPLB_TUNING
+  {
+    hipFuncAttributes attr;
+    (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
+    fprintf(stderr, "plan variant <%d,%d,%d,K=%d,W=%d>: %d workgroups, lds %zu, %d fit a CU, %d CUs (numRegs %d, static LDS %zu)\n",
+            GM, DM, (int)EXACT, K, WAVES, n_workgroups, lds, fit, d->n_cus, attr.numRegs, attr.sharedSizeBytes);
+  }
+#endif
+  if (fit <= 0 || n_workgroups > (int)(kResidencyBudget * fit * d->n_cus))
+    return LPLB_OK;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capture) != hipSuccess)
+    capture = hipStreamCaptureStatusNone;
+  const bool capturing = capture == hipStreamCaptureStatusActive;
+  const float cost = (float)n_workgroups / (float)(fit * d->n_cus);
+  std::lock_guard<std::mutex> lock(g_plan_guard);   // held over the launch: admission and launch order agree
+  const int slot = admit_launch(*d, s, cost, capturing);
+#ifdef LPLB_TUNING
+  fprintf(stderr, "  admission: slot %d, cost %.3f\n", slot, cost);
+#endif
+  if (slot < 0)
+    return LPLB_OK;
+  PlanSlot &ps = d->slots[slot];
+  a.sync = d->sync + (size_t)slot * kSlotInts;
+  a.solve.tagged_result = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
+  a.expected_slices = a.n_slices + g_fault_extra_slices.exchange(0);
+  const int fault_polls = g_fault_max_polls.exchange(0);
+  a.max_polls = fault_polls > 0 ? fault_polls : kDefaultMaxPolls;
+  launch(kernel, dim3(n_workgroups), dim3(WAVES * kWave), lds, s, a);
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess)
+    return fail(LPLB_EHIP, "plan: launch failed: %s", hipGetErrorString(err));
+  ps.maybe_executing = !capturing;
+  g_one_launch_plans.fetch_add(1, std::memory_order_relaxed);
+  *done = true;
+  return LPLB_OK;
+}
+
+// Chunks per wave (1, 2, 4, 8 or 16) that cover a slice of `per` indices with `waves` waves.
+static int chunks_per_wave(int64_t per, int waves) {
+  const int64_t chunks = (per + kWave - 1) / kWave;
+  const int64_t needed = (chunks + waves - 1) / waves;
+  return needed <= 1 ? 1 : needed <= 2 ? 2 : needed <= 4 ? 4 : needed <= 8 ? 8 : 16;
+}
+
+template <int GM, int DM, bool EXACT, int W>
+static int launch_plan_shape(PlanArgs &a, hipStream_t s, bool *done) {
+  const int k = chunks_per_wave(a.per, W);
+  const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, a.n_rep, W, k);
+  const size_t lds_lp = (size_t)min(a.solve.n_units, kLpsPerWorkgroup) * a.solve.n_experts * sizeof(float);
+  if (lds_slices > (size_t)kPlanLdsLimit)
+    return LPLB_OK;
+  a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
+  if (a.local_counts && (size_t)a.solve.n_experts * sizeof(float) > lds_slices)
+    return LPLB_OK;   // the LP takes its counts from LDS in that mode
+  switch (k) {
+  case 1: return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s, done);
+  case 2: return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds_slices, s, done);
+  case 4: return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s, done);
+  case 8: return launch_plan_variant<GM, DM, EXACT, 8, W>(a, lds_slices, s, done);
+  default:
+    if constexpr (W == 8)
+      return launch_plan_variant<GM, DM, EXACT, 16, W>(a, lds_slices, s, done);
+    return LPLB_OK;
+  }
+}
+
+// Tries the one-launch plan.  *done = false: shape or size outside what it covers, or no
+// room on the GPU right now; nothing was enqueued.
 static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t *counts, const int32_t *r2o,
                           const int32_t *o2r, const int32_t *phy2log, int n_group, int G, int D, int C, int P,
                           int n_blocks, int32_t *counts_by_block, float *global_workload, float *o_weight,
@@ -501,72 +822,75 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
                           hipStream_t s, bool *done) {
   *done = false;
   const int L = P - D * C, n_fixed = L - D * C;
-  const int n_logical = n_group * G * L;
+  const int n_logical = n_group * G * L, n_rep = n_group * G * C * D;
   if (!g_cooperative || n_elements <= 0 || n_blocks < 2)
     return LPLB_OK;
   int gm = 0, dm = 0;
   if (!plan_lp_shape(G, D, &gm, &dm) || n_group > kLpsPerWorkgroup * kMaxLpWorkgroups ||
-      n_group * G * D > kMaxShares || global_workload == nullptr)
+      n_group * G * D > kMaxShares || global_workload == nullptr || n_logical > kMaxTotals ||
+      n_group * G * P >= 65536 || n_elements > (INT32_MAX - 41) / 499)
     return LPLB_OK;
-  // Shapes built for 16 waves also exist with 8: a slice workgroup's LDS grows with
-  // waves x logical experts, and from about 400 experts on only 8 waves fit.
-  int waves = plan_waves(gm, dm);
-  if (waves == 16 && plan_lds_bytes(n_logical, 16) > (size_t)kPlanLdsLimit)
-    waves = 8;
   const int n_lp_workgroups = (n_group + kLpsPerWorkgroup - 1) / kLpsPerWorkgroup;
-  // own-histogram mode: the totals fit the accumulator (and with it the LDS)
-  if (counts == nullptr && n_logical > kMaxTotals)
+  const int n_cus = current_device_cu_count();
+  if (n_cus <= 0)
     return LPLB_OK;
-  // slices of 1024 indices while kMaxSlices of them cover the batch, else of 2048, 4096,
-  // 8192; at most n_blocks - 1 of them (the caller's bound on parallelism; the last row of
-  // its table takes the totals)
-  int64_t slices = kMaxSlices + 1;
-  for (int64_t len = 1024; len <= (int64_t)waves * kChunksPerWave * kWave && slices > kMaxSlices; len *= 2)
-    slices = (n_elements + len - 1) / len;
-  if (slices > kMaxSlices)
-    return LPLB_OK;
+  // Workgroup size: 16 waves where the LP's registers allow it, 8 where they do not, where
+  // the LDS tables need it, and for batches so long that 16-wave workgroups (one per CU)
+  // could not all be resident.
+  int waves = plan_waves(gm, dm);
+  // Slices of 1024 indices while kPreferredSlices of them cover the batch, else of 2048,
+  // 4096, 8192 (the longest a workgroup holds in registers); at most n_blocks - 1 of them
+  // (the caller's bound on parallelism; the last row of its table takes the totals).
+  const int64_t longest = 8192;
+  int64_t len = 1024;
+  while (len < longest && (n_elements + len - 1) / len > kPreferredSlices)
+    len *= 2;
+  int64_t slices = (n_elements + len - 1) / len;
   if (slices > n_blocks - 1)
     slices = n_blocks - 1;
   const int64_t per = slice_len(n_elements, (int)slices);
-  if (per > (int64_t)waves * kChunksPerWave * kWave || plan_lds_bytes(n_logical, waves) > (size_t)kPlanLdsLimit)
+  if (per > longest)
     return LPLB_OK;
-  int *sync = nullptr, n_cus = 0;
-  int rc = plan_device_state(&sync, &n_cus);
-  if (rc != LPLB_OK)
-    return rc;
-  const int slot = sync_slot_of(s);
-  // a quarter of the CUs for the slices, so that three plans that execute at once are all resident
-  if (slices > n_cus / 4 || slot < 0)
-    return LPLB_OK;
-  sync += (size_t)slot * kSlotInts;
+  slices = (n_elements + per - 1) / per;   // (rounding the slice length up may have emptied the last ones)
+  if (waves == 16 && (slices + n_lp_workgroups > n_cus / 2 ||
+                      plan_lds_bytes(n_logical, n_rep, 16, chunks_per_wave(per, 16)) > (size_t)kPlanLdsLimit))
+    waves = 8;
+  int row_shift = 0;
+  while ((1 << row_shift) < n_rep)
+    ++row_shift;
+  if ((slices << row_shift) > (int64_t)(n_blocks - 1) * n_logical)
+    return LPLB_OK;   // the rows of the exchange live in the caller's table
 
   PlanArgs a{};   // every field the host does not set below is zero
   a.idx = idx; a.n = n_elements; a.per = per; a.n_slices = (int)slices; a.n_lp_workgroups = n_lp_workgroups;
-  a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block;
+  a.o2r = o2r; a.phy2log = phy2log; a.rows = counts_by_block; a.row_shift = row_shift;
   a.totals = counts_by_block + (int64_t)(n_blocks - 1) * n_logical; a.out = out;
-  a.physical_counts = physical_counts;
+  a.physical_counts = physical_counts; a.avail = avail_num;
   a.sh = RedirectShape{n_logical, n_group * G, G, D, C, L, P};
-  a.local_counts = counts == nullptr; a.sync = sync;
+  a.n_rep = n_rep;
+  a.magic_L = fast_div_magic((uint32_t)L); a.magic_cd = fast_div_magic((uint32_t)(C * D));
+  a.magic_D = fast_div_magic((uint32_t)D); a.magic_G = fast_div_magic((uint32_t)G);
+  a.local_counts = counts == nullptr;
+  a.n_copies = 1;
+  while (a.n_copies < kTotalCopies && a.n_copies * 16 < a.n_slices)
+    a.n_copies *= 2;
   SolveArgs &sa = a.solve;
   sa.workload = counts; sa.gw_out = global_workload; sa.r2o = r2o; sa.phy2log = phy2log;
   sa.avail = avail_num; sa.result = o_weight; sa.n_group = n_group; sa.G = G; sa.D = D; sa.C = C;
   sa.n_fixed = n_fixed; sa.n_experts = n_logical; sa.step_rule = step_rule; sa.n_steps = n_steps;
   sa.n_units = n_group; sa.staged_stride = 0;
-  sa.tagged_result = reinterpret_cast<unsigned long long *>(sync + kSharesAt);
   sa.clocks = debug_clocks();
 
-  hipError_t err = hipErrorInvalidValue;
+  int rc = LPLB_OK;
 #define LPLB_PLAN_CASE_W(GM, DM, W)                                                            \
   if (gm == GM && dm == DM && waves == W)                                                      \
-    err = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true, W>(a, s)                     \
-                               : launch_plan_shape<GM, DM, false, W>(a, s);
+    rc = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true, W>(a, s, done)                \
+                              : launch_plan_shape<GM, DM, false, W>(a, s, done);
   LPLB_PLAN_CASE_W(8, 1, 16) LPLB_PLAN_CASE_W(8, 1, 8) LPLB_PLAN_CASE_W(8, 2, 16) LPLB_PLAN_CASE_W(8, 2, 8)
   LPLB_PLAN_CASE_W(8, 4, 8) LPLB_PLAN_CASE_W(16, 1, 16) LPLB_PLAN_CASE_W(16, 1, 8) LPLB_PLAN_CASE_W(16, 2, 8)
   LPLB_PLAN_CASE_W(32, 1, 8) LPLB_PLAN_CASE_W(32, 2, 8)
 #undef LPLB_PLAN_CASE_W
-  LPLB_HIP_TRY(err);
-  *done = true;
-  return LPLB_OK;
+  return rc;
 }
 
 } // namespace lplb
@@ -579,16 +903,29 @@ extern "C" int lplb_plan_set_cooperative(int enabled) {
 extern "C" int lplb_plan_sync_timeouts(int *count) {
   using namespace lplb;
   LPLB_REQUIRE(count != nullptr, LPLB_EINVAL, "plan_sync_timeouts: null pointer");
-  int *sync = nullptr, n_cus = 0;
-  int rc = plan_device_state(&sync, &n_cus);
+  PlanDevice *d = nullptr;
+  const int rc = plan_device(&d);
   if (rc != LPLB_OK)
     return rc;
   *count = 0;
   for (int slot = 0; slot < kSyncSlots; ++slot) {
     int n = 0;
-    LPLB_HIP_TRY(hipMemcpy(&n, sync + (size_t)slot * kSlotInts + 3, sizeof(int), hipMemcpyDeviceToHost));
+    LPLB_HIP_TRY(hipMemcpy(&n, d->sync + (size_t)slot * kSlotInts + kTimeoutsAt, sizeof(int), hipMemcpyDeviceToHost));
     *count += n;
   }
+  return LPLB_OK;
+}
+
+extern "C" int lplb_plan_one_launch_count(long long *count) {
+  LPLB_REQUIRE(count != nullptr, LPLB_EINVAL, "plan_one_launch_count: null pointer");
+  *count = lplb::g_one_launch_plans.load(std::memory_order_relaxed);
+  return LPLB_OK;
+}
+
+extern "C" int lplb_plan_inject_fault(int extra_slices_expected, int max_polls) {
+  LPLB_REQUIRE(extra_slices_expected >= 0 && max_polls >= 0, LPLB_EINVAL, "plan_inject_fault: negative argument");
+  lplb::g_fault_extra_slices = extra_slices_expected;
+  lplb::g_fault_max_polls = max_polls;
   return LPLB_OK;
 }
 

@@ -48,6 +48,7 @@ struct SolveArgs {
                              // wave's LP into staged_counts (as floats) and a.workload is not read
   unsigned long long *tagged_result;  // or null: a copy of a.result for other workgroups of the same launch,
                                       // each value written through to memory as (1 << 32) | its bits
+                                      // (tag 2 instead of 1 means "no result: use the neutral fallback")
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
 
@@ -185,7 +186,8 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, int64_t
 //   staged_counts  LDS, ROWS * a.staged_stride floats (unused if the stride is 0)
 //   rep_of_edge    LDS, kWave ints
 // Returns how many of the wave's LPs passed the feasibility test (same value in
-// every lane); the caller adds it to a.avail.
+// every lane); the caller adds it to a.avail.  -1: the counts the caller promised through
+// a.counts_ready never came; nothing was solved or stored.
 template <int GM, int DM, bool EXACT, int ROWS>
 __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged_counts_of_wave,
                                int *rep_of_edge) {
@@ -253,8 +255,17 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   float wmax = 0.0f;
   float out_cnt[KG];
   if (prestaged) {
-    while (__hip_atomic_load(a.counts_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0)
+    // 1 = the counts are staged, 2 = the caller gave up on them; the wait itself is bounded
+    // as well (2^26 polls, seconds), so that this wave ends whatever happens to the flag.
+    int ready = 0;
+    for (int polls = 0; polls < (1 << 26); ++polls) {
+      ready = __hip_atomic_load(a.counts_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (ready != 0)
+        break;
       __builtin_amdgcn_s_sleep(1);
+    }
+    if (ready != 1)
+      return -1;   // nothing has been written
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     for (int i = lane; i < a.n_experts; i += WL)
       wmax = fmaxf(wmax, staged_counts[i]);

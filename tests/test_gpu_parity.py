@@ -746,7 +746,7 @@ def test_plan_one_launch_equals_chain(cuda, cfg, use_global, tokens, n_sms):
     """Short batches run as one kernel launch whose workgroups exchange histogram rows and the
     LP's shares through memory; the result must be the chain's, bit for bit, call after call."""
     inp = synth.make_inputs(cfg, tokens=tokens, mask_fraction=0.05) if tokens else synth.make_inputs(cfg, mask_fraction=0.05)
-    _one_launch_equals_chain(cuda, inp, use_global, n_sms)
+    _one_launch_equals_chain(cuda, inp, use_global, n_sms, expect_one_launch=True)
 
 
 MANY_GROUPS = {
@@ -772,7 +772,7 @@ def test_plan_one_launch_with_many_groups(cuda, name, use_global):
     inp = synth.make_inputs(MANY_GROUPS[name], mask_fraction=0.02)
     c = inp.cfg
     shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
-    got = _one_launch_equals_chain(cuda, inp, use_global, 256)
+    got = _one_launch_equals_chain(cuda, inp, use_global, 256, expect_one_launch=True)
     # and the chain's result is the oracle's
     counts = inp.global_counts if use_global else np.bincount(inp.indices[inp.indices >= 0].ravel(),
                                                               minlength=c.n_logical).astype(np.int32)
@@ -784,8 +784,12 @@ def test_plan_one_launch_with_many_groups(cuda, name, use_global):
     np.testing.assert_array_equal(got[0], want)
 
 
-def _one_launch_equals_chain(cuda, inp, use_global, n_sms):
+def _one_launch_equals_chain(cuda, inp, use_global, n_sms, expect_one_launch=None):
+    """Runs the plan as the chain, then twice in the default mode; everything must agree bit for bit.
+    expect_one_launch=True additionally requires that the default mode really ran as one kernel launch
+    (the library counts those), so that the comparison is not the chain against itself."""
     from lplb_amd import _native
+    timeouts_before = _native.plan_sync_timeouts()
     c = inp.cfg
     shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
     solver = solver_for(shape)
@@ -798,9 +802,14 @@ def _one_launch_equals_chain(cuda, inp, use_global, n_sms):
             _native.set_plan_cooperative(mode)
             avail = torch.zeros(1, dtype=torch.int32, device=cuda)
             phys = torch.full((shape.n_physical,), -7, dtype=torch.int32, device=cuda)
+            launches_before = _native.plan_one_launch_count()
             out, o_weight, by_sm = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, n_sms,
                                                global_counts=counts, physical_counts=phys)
             torch.cuda.synchronize()
+            as_one_launch = _native.plan_one_launch_count() - launches_before
+            assert as_one_launch == 0 if not mode else as_one_launch in (0, 1)
+            if mode and expect_one_launch is not None:
+                assert as_one_launch == int(expect_one_launch), "the plan did not take the expected form"
             got = (out.cpu().numpy(), o_weight.cpu().numpy(), by_sm[-1].cpu().numpy(), int(avail[0]),
                    phys.cpu().numpy())
             if mode not in runs:
@@ -809,7 +818,7 @@ def _one_launch_equals_chain(cuda, inp, use_global, n_sms):
                 np.testing.assert_array_equal(a, b)
     finally:
         _native.set_plan_cooperative(True)
-    assert _native.plan_sync_timeouts() == 0
+    assert _native.plan_sync_timeouts() == timeouts_before
     np.testing.assert_array_equal(runs[True][2], np.bincount(inp.indices[inp.indices >= 0].ravel(),
                                                              minlength=c.n_logical))
     out = runs[True][0]
@@ -823,6 +832,7 @@ def test_plan_random_shapes_one_launch_equals_chain(cuda):
     from lplb_amd import _native, topology
     from lplb_amd.mapping import build_redundancy_mapping
     rng = np.random.default_rng(77)
+    timeouts_before = _native.plan_sync_timeouts()
     topologies = [(topology.CUBE_8P2E, 1), (topology.RING_8P, 1), (topology.HYPERCUBE_16P2E, 1),
                   (topology.torus_2d(8, 4), 1), (topology.CUBE_8P2E, 4), (_shifted_ring(6, [1, 2]), 2),
                   (_shifted_ring(4, [1, 2, 3]), 3), (_shifted_ring(16, [1]), 2), (topology.CUBE_8P2E, 9),
@@ -862,7 +872,7 @@ def test_plan_random_shapes_one_launch_equals_chain(cuda):
                     np.testing.assert_array_equal(a, b, err_msg=f"trial {trial} {r2o.shape} n={n} n_sms={n_sms}")
     finally:
         _native.set_plan_cooperative(True)
-    assert _native.plan_sync_timeouts() == 0
+    assert _native.plan_sync_timeouts() == timeouts_before
 
 
 def test_planner_run_equals_plan_with_local_counts(cuda):
@@ -996,8 +1006,7 @@ def test_planner_run_replays_from_a_hip_graph(cuda):
 @pytest.mark.parametrize("cooperative", [False, True])
 def test_plans_on_two_streams(cuda, cooperative):
     """Plans on different streams may overlap on the device.  The one-launch form keeps its
-    counters per stream (for the first two streams that plan; later ones get the chain), and the
-    chain of kernels has no shared state at all."""
+    counters per stream, and the chain of kernels has no shared state at all."""
     from lplb_amd import _native
     inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
     other = synth.make_inputs("v3_ep8_cube", tokens=5000, mask_fraction=0.1)
@@ -1007,6 +1016,7 @@ def test_plans_on_two_streams(cuda, cooperative):
     want_b, _, _ = solver.plan(idx_b, t["r2o"], t["o2r"], t["phy2log"], avail, 256)
     torch.cuda.synchronize()
     streams = [torch.cuda.current_stream(), torch.cuda.Stream(), torch.cuda.Stream()]
+    timeouts_before, launches_before = _native.plan_sync_timeouts(), _native.plan_one_launch_count()
     _native.set_plan_cooperative(cooperative)
     try:
         for rep in range(30):
@@ -1016,7 +1026,9 @@ def test_plans_on_two_streams(cuda, cooperative):
                     outs.append(solver.plan(idx, t["r2o"], t["o2r"], t["phy2log"], avail, 256)[0])
             torch.cuda.synchronize()
             assert torch.equal(outs[0], want_a) and torch.equal(outs[1], want_b) and torch.equal(outs[2], want_a), rep
-        assert _native.plan_sync_timeouts() == 0
+        assert _native.plan_sync_timeouts() == timeouts_before
+        # three plans of 65 workgroups fit the GPU side by side: all 90 ran as one launch each (or none)
+        assert _native.plan_one_launch_count() - launches_before == (90 if cooperative else 0)
     finally:
         _native.set_plan_cooperative(True)
 
@@ -1033,6 +1045,7 @@ def test_one_launch_plan_while_another_stream_fills_the_gpu(cuda):
     a = torch.randn(4096, 4096, device=cuda, dtype=torch.bfloat16)
     b = torch.randn(4096, 4096, device=cuda, dtype=torch.bfloat16)
     busy, planning = torch.cuda.Stream(), torch.cuda.Stream()
+    timeouts_before, launches_before = _native.plan_sync_timeouts(), _native.plan_one_launch_count()
     for rep in range(10):
         with torch.cuda.stream(busy):
             for _ in range(4):
@@ -1043,7 +1056,112 @@ def test_one_launch_plan_while_another_stream_fills_the_gpu(cuda):
         torch.cuda.synchronize()
         assert all(torch.equal(o, want) for o in outs), rep
         del c
-    assert _native.plan_sync_timeouts() == 0
+    assert _native.plan_sync_timeouts() == timeouts_before
+    assert _native.plan_one_launch_count() - launches_before == 40     # not the chain by accident
+
+
+@pytest.mark.parametrize("use_global", [True, False])
+def test_plan_at_the_sweep_shape_is_one_launch_and_equals_the_chain(cuda, use_global):
+    """[262144 x 8] indices: 256 slices of 8192 indices (16 chunks per wave) and the LP in one grid."""
+    inp = synth.make_inputs("sweep_redirect", mask_fraction=0.01)
+    got = _one_launch_equals_chain(cuda, inp, use_global, 512, expect_one_launch=True)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    by_sm = oracle.count_idx(inp.indices.reshape(-1), c.n_logical, 512)
+    want = oracle.map_idx(inp.indices.reshape(-1), got[1], by_sm, shape.o2r, inp.phy2log, shape.n_group, shape.C,
+                          shape.P).reshape(inp.indices.shape)
+    np.testing.assert_array_equal(got[0], want)
+
+
+@pytest.mark.parametrize("use_global", [True, False])
+def test_one_launch_plan_gives_up_in_a_defined_way(cuda, use_global):
+    """A wait between workgroups that cannot be met (forced from the host: the kernel is told to expect
+    one slice more than its grid has, and to poll 2000 times instead of millions) must end in the
+    documented fallback -- every token on its expert's original slot, the feasible-LP counter untouched,
+    physical_counts filled with -1, the give-ups counted -- with every kernel ending normally, and
+    the next plan on the same stream must be right again (minilp.cu:395-397 is the reference's own
+    neutral fallback for an LP that fails)."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    lib = _native.load()
+    counts = t["counts"] if use_global else None
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    phys = torch.full((shape.n_physical,), -7, dtype=torch.int32, device=cuda)
+    want, want_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
+                                  physical_counts=phys)
+    want, want_w, want_phys = want.clone(), want_w.clone(), phys.clone()
+    torch.cuda.synchronize()
+    assert int(avail[0]) == 1
+    timeouts_before, launches_before = _native.plan_sync_timeouts(), _native.plan_one_launch_count()
+    print("injecting a wait that cannot be met", flush=True)
+    assert lib.lplb_plan_inject_fault(1, 2000) == 0
+    out, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
+                            physical_counts=phys)
+    torch.cuda.synchronize()
+    assert _native.plan_one_launch_count() == launches_before + 1
+    # the fallback: the redirect with every share = 1 keeps every token on the original
+    by_sm = oracle.count_idx(inp.indices, shape.n_logical, 256)
+    stay = oracle.map_idx(inp.indices, np.ones((1, shape.G, shape.D), np.float32), by_sm, shape.o2r, inp.phy2log, 1,
+                          shape.C, shape.P)
+    np.testing.assert_array_equal(out.cpu().numpy(), stay)
+    assert int(avail[0]) == 1                       # withheld
+    assert torch.all(phys == -1)
+    gave_up = _native.plan_sync_timeouts() - timeouts_before
+    assert gave_up >= 64, gave_up                   # every slice workgroup's wait (and the LP's, if it waited too)
+    # the next plans on the same stream are healthy
+    for _ in range(3):
+        out, o_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
+                                  physical_counts=phys)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(o_w, want_w) and torch.equal(phys, want_phys)
+    assert int(avail[0]) == 4
+    assert _native.plan_sync_timeouts() - timeouts_before == gave_up
+    assert _native.plan_one_launch_count() == launches_before + 4
+
+
+def test_one_launch_slots_pass_from_stream_to_stream(cuda):
+    """More streams than the library has counter blocks: a block whose last launch has completed
+    passes to the next stream, so a long-running process keeps the one-launch form."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)
+    want = want.clone()
+    torch.cuda.synchronize()
+    launches_before = _native.plan_one_launch_count()
+    streams = [torch.cuda.Stream() for _ in range(20)]
+    for s_ in streams:
+        s_.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s_):
+            out, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)
+        s_.synchronize()
+        assert torch.equal(out, want)
+    assert _native.plan_one_launch_count() - launches_before == 20
+
+
+def test_one_launch_plans_beyond_what_fits_the_gpu_run_as_the_chain(cuda):
+    """Twelve streams plan at the same time without waiting for each other.  Only as many one-launch
+    plans as fit the GPU side by side are admitted (their workgroups wait for each other); the rest
+    run as the chain.  Every result is right and no wait runs out."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)
+    want = want.clone()
+    torch.cuda.synchronize()
+    timeouts_before, launches_before = _native.plan_sync_timeouts(), _native.plan_one_launch_count()
+    streams = [torch.cuda.Stream() for _ in range(12)]
+    for rep in range(5):
+        outs = []
+        for s_ in streams:
+            with torch.cuda.stream(s_):
+                outs.append(solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256)[0])
+        torch.cuda.synchronize()
+        assert all(torch.equal(o, want) for o in outs), rep
+    as_one_launch = _native.plan_one_launch_count() - launches_before
+    print(f"{as_one_launch} of 60 concurrent plans ran as one launch")
+    assert 5 <= as_one_launch <= 60
+    assert _native.plan_sync_timeouts() == timeouts_before
 
 
 def test_kernel_timestamp_hook(cuda):

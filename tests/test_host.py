@@ -190,7 +190,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert sorted(_native.exported_symbols()) == declared
-    assert lib.lplb_abi_version() == _native.ABI_VERSION == 3
+    assert lib.lplb_abi_version() == _native.ABI_VERSION == 4
     header = (ROOT / "include" / "lplb_hip.h").read_text()
     assert f"#define LPLB_ABI_VERSION {_native.ABI_VERSION}" in header
 
@@ -221,3 +221,53 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.lplb_plan(p, 5_000_000, None, p, p, p, 1, 8, 2, 1, 34, 256, p, p, p, p, p, p, 0, 5, None) == 2
     assert b"physical_counts" in lib.lplb_last_error()
     assert lib.lplb_map_idx(p, p, p, p, p, 5_000_000, 1, 8, 2, 1, 34, 256, p, p, None) == 2
+
+
+def test_cross_workgroup_helpers_compile_to_the_forms_the_plan_relies_on(tmp_path):
+    """The workgroups of the one-launch plan exchange data through agent-scope atomics
+    (lplb_amd/csrc/plan_sync.h).  That works across the GPU's eight L2 caches because those
+    atomics bypass the L2 (sc1 bit), the acquire fence invalidates it (buffer_inv sc1) and
+    s_waitcnt vmcnt(0) waits for the stores' acknowledgement.  Compile the helpers on their own
+    and look at what the compiler makes of them, so that a toolchain that lowers them
+    differently fails here and not silently on the GPU."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(hipcc).exists():
+        pytest.skip("no hipcc")
+    probe = tmp_path / "probe.hip"
+    probe.write_text('''
+#include "plan_sync.h"
+using namespace lplb;
+extern "C" __global__ void publish(int *row, unsigned long long *word, int *counter) {
+  agent_store(row + threadIdx.x, 7);
+  agent_add(word, (5ull << 32) | 1ull);
+  stores_have_landed();
+  __syncthreads();
+  if (threadIdx.x == 0)
+    announce_arrival(counter, blockIdx.x);
+}
+extern "C" __global__ void consume(int *counter, const int *row, const unsigned long long *word, int *out) {
+  if (threadIdx.x < 64)
+    out[64] = wait_for_arrivals(counter, 3, 1000);
+  __syncthreads();
+  out[threadIdx.x] = row[threadIdx.x] + (int)(agent_load(word) >> 32);
+}
+''')
+    asm = tmp_path / "probe.s"
+    subprocess.run([hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "--cuda-device-only", "-S",
+                    f"-I{ROOT / 'lplb_amd' / 'csrc'}", str(probe), "-o", str(asm)], check=True, capture_output=True)
+    text = asm.read_text()
+    publish, consume = text.split("consume:")[0], text.split("consume:")[1]
+    assert re.search(r"global_store_dword .* sc1", publish), "agent-scope store does not write through"
+    # read-modify-writes are carried out by the atomic unit behind the caches (no cached copy to go stale)
+    assert "global_atomic_add_x2" in publish and re.search(r"global_atomic_add v", publish)
+    # the row's stores are acknowledged before the barrier that precedes the counter update
+    body = publish[publish.index("global_store_dword"):]
+    assert body.index("s_waitcnt vmcnt(0)") < body.index("s_barrier") < body.rindex("global_atomic_add v")
+    assert re.search(r"global_load_dword .* sc1", consume), "agent-scope load may hit a stale L2 line"
+    assert "buffer_inv sc1" in consume, "the acquire fence does not invalidate the L2"
+    # the polls come before the invalidate, the plain read of the row after it
+    polls, after_fence = consume.split("buffer_inv sc1")
+    assert "s_sleep" in polls and re.search(r"global_load_dword v\d+, v\d+, s\[\d+:\d+\]\n", after_fence)
+    assert re.search(r"global_load_dwordx2 .* sc1", after_fence), "the tagged word is read past the L2"
