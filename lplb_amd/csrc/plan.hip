@@ -19,14 +19,19 @@
 //   LP workgroup: (own-histogram mode: wait for the totals ->) solve -> publish the shares.
 // What crosses workgroups is written and read with agent-scope atomics (plan_sync.h).
 // The workgroups wait for each other, so the whole grid has to be resident: its size is
-// bounded by what the occupancy query says fits the GPU, and the host admits a launch
-// only while the plans still executing leave room for it (it asks the runtime whether the
-// streams that planned last still have work pending; it never waits); everything else
-// runs as the chain.  Every wait
-// is bounded all the same.  A wait that runs out is counted and the launch degrades
-// in a defined way: every token of the affected slices goes to its expert's original
-// slot (which needs nothing from other workgroups), the feasible-LP counter is left
-// alone and physical_counts, if asked for, is filled with -1.
+// bounded by what fits the GPU, and the host admits a launch only while the plans still
+// executing leave room for it (it asks the runtime whether the streams that planned last
+// still have work pending; it never waits); everything else runs as the chain.
+// Nothing is cleared at the end of a launch (finding out which workgroup is the last costs
+// two more round trips through memory on the critical path): a launch counter in device
+// memory tags the shares and selects one of two sets of counters, and every launch clears,
+// while it waits for its indices, the set that the launch before it used.
+// Every wait is bounded all the same.  A wait that runs out is counted, the workgroup sends
+// every token of its slice to the expert's original slot (which needs nothing from other
+// workgroups), physical_counts is filled with -1 by the workgroup that writes them if it
+// is among those, and the block of counters is marked as unusable: plans that use it later
+// send every token to the original slot and count one more failure each, until
+// lplb_plan_sync_timeouts has reported the failures and cleared the block.
 #include "map_kernel.h"
 #include "plan_sync.h"
 #include "solve_kernel.h"
@@ -46,25 +51,27 @@ constexpr int kDefaultMaxPolls = 1 << 22;   // a few seconds of polling before a
 constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 
 // One block of these per stream that plans (kSyncSlots of them per device):
-//   [kArrivedAt ..] slices that have published their counts (striped), [kLeftStripesAt ..] and
-//   [kLeftAt] workgroups that need nothing from the others any more (see leave());
-//   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits, tag 0 = not
-//   there yet, 1 = valid, 2 = there will be none;
-//   from kTotalsAt: partial histograms of the batch, [copy][n_logical] 8-byte words with the
-//   tokens in the high half and the number of slices that have contributed in the low half
-//   (one atomic add delivers both, so whoever polls the words needs no second round trip
-//   for a "done" counter).  Slice s adds its histogram to copy s % n_copies: updates of one
-//   address queue up behind each other, about 35 ns each, so one copy per 16 slices (at most
-//   kTotalCopies); whoever needs the batch's tokens per expert adds the copies up.
-// The last workgroup to leave clears the block, so a captured launch can be replayed.
-constexpr int kLeftAt = 1;
-// ... and one that is never cleared: waits that ran out since the library was loaded
-constexpr int kTimeoutsAt = 4;
-constexpr int kArrivedAt = 16;      // kArrivalStripes words, one 64-byte line
-constexpr int kLeftStripesAt = 32;  // kArrivalStripes words: workgroups that have left, first level
+//   [kGenAt] launches that have completed their exchange of counts; its parity p selects the
+//   set of counters a launch uses, and (value + 1) tags what the LP publishes;
+//   [kPoisonAt] non-zero: a wait ran out in this block (see above); [kTimeoutsAt] waits that
+//   ran out since the library was loaded (never cleared);
+//   [kDirtyAt + p] how many words of set p's totals the last launch that used it may have left non-zero;
+//   [kArrivedAt + 16 p ..] workgroups that have published (slices) or started (LP), striped;
+//   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits with
+//   tag = (launch tag << 2) | 1 (valid) or 2 (there will be none); a word with another
+//   launch's tag is "not there yet";
+//   from kTotalsAt: two sets of partial histograms of the batch, [p][copy][n_logical] 8-byte
+//   words with the tokens in the high half and the number of slices that have contributed in
+//   the low half (one atomic add delivers both, so whoever polls the words needs no second
+//   round trip for a "done" counter).  Slice s adds its histogram to copy s % n_copies:
+//   updates of one address queue up behind each other, about 35 ns each, so one copy per 16
+//   slices (at most kTotalCopies); whoever needs the batch's tokens per expert adds the copies up.
+constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8;
+constexpr int kArrivedAt = 16;      // 2 x kArrivalStripes words, a 64-byte line each
 constexpr int kSharesAt = 48, kMaxShares = 1024;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024, kTotalCopies = 16;
-constexpr int kSlotInts = kTotalsAt + 2 * kTotalCopies * kMaxTotals, kSyncSlots = 8;
+constexpr int kTotalsWords = kTotalCopies * kMaxTotals;   // 8-byte words of one set
+constexpr int kSlotInts = kTotalsAt + 2 * 2 * kTotalsWords, kSyncSlots = 8;
 static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
 static std::atomic<bool> g_cooperative{true};   // any thread may flip it while others plan
 static std::atomic<long long> g_one_launch_plans{0};
@@ -94,67 +101,10 @@ struct PlanArgs {
   int *sync;
 };
 
-// A wait ran out: count it (the workgroup also says so when it leaves).
-__device__ inline void give_up(const PlanArgs &a) { agent_add(a.sync + kTimeoutsAt, 1); }
-
-// Called by a whole workgroup when it needs nothing from the others any more.  The last of
-// the grid's workgroups to get here adds the feasible LPs to the caller's counter (unless a
-// wait ran out) and clears the block for the next launch (which starts after this kernel
-// has ended, so the clearing stores need no wait of their own).
-// Who is last is counted in two levels (updates of one address queue up, about 35 ns each):
-// the last of the workgroups that share a stripe counts for the stripe, the last stripe is
-// last.  What the last one has to know travels in the counters themselves: bits 0-11 count
-// workgroups or stripes, bits 12-23 those of them in which a wait ran out, bits 24-31 feasible LPs.
-// gave_up / feasible: LDS words of this workgroup, read after its waves have met.
-__device__ inline void leave(const PlanArgs &a, int n_shares, const int *gave_up, const int *feasible) {
-  __shared__ int last_to_leave, summary;
-  const int nl = a.sh.n_logical;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int n_workgroups = a.n_slices + a.n_lp_workgroups;
-    const int stripe = blockIdx.x % kArrivalStripes;
-    const int in_stripe = (n_workgroups - stripe + kArrivalStripes - 1) / kArrivalStripes;
-    const int mine = 1 + ((*gave_up ? 1 : 0) << 12) + (*feasible << 24);
-    const int of_stripe = agent_add(a.sync + kLeftStripesAt + stripe, mine) + mine;
-    last_to_leave = 0;
-    if ((of_stripe & 0xfff) == in_stripe) {
-      const int up = 1 + (((of_stripe >> 12) & 0xfff ? 1 : 0) << 12) + (of_stripe & 0xff000000);
-      const int all = agent_add(a.sync + kLeftAt, up) + up;
-      last_to_leave = (all & 0xfff) == min(n_workgroups, kArrivalStripes);
-      summary = all;
-    }
-  }
-  __syncthreads();
-  if (!last_to_leave)
-    return;
-#ifdef LPLB_PHASE_CLOCKS
-  if (a.solve.clocks && threadIdx.x == 0)
-    a.solve.clocks[112] = wall_clock64();
-#endif
-  const bool failed = ((summary >> 12) & 0xfff) != 0;
-  unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
-  unsigned long long *totals = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt);
-  for (int i = threadIdx.x; i < a.n_copies * nl; i += blockDim.x)
-    agent_store(totals + i, 0ull);
-  for (int i = threadIdx.x; i < n_shares; i += blockDim.x)
-    agent_store(shares + i, 0ull);
-  if (threadIdx.x < kArrivalStripes) {
-    agent_store(a.sync + kArrivedAt + threadIdx.x, 0);
-    agent_store(a.sync + kLeftStripesAt + threadIdx.x, 0);
-  }
-  if (failed && a.physical_counts)
-    for (int i = threadIdx.x; i < a.sh.n_ranks * a.sh.P; i += blockDim.x)
-      a.physical_counts[i] = -1;
-  if (threadIdx.x == 0) {
-    const int n_feasible = (int)((unsigned)summary >> 24);
-    if (!failed && n_feasible > 0)
-      atomicAdd(a.avail, n_feasible);
-    agent_store(a.sync + kLeftAt, 0);
-#ifdef LPLB_PHASE_CLOCKS
-    if (a.solve.clocks)
-      a.solve.clocks[113] = wall_clock64();
-#endif
-  }
+// A wait ran out: count it and switch the block of counters off.
+__device__ inline void give_up(const PlanArgs &a) {
+  agent_add(a.sync + kTimeoutsAt, 1);
+  agent_store(a.sync + kPoisonAt, 1);
 }
 
 // LDS of a slice workgroup: route and histogram per logical expert, a ranking record per
@@ -180,17 +130,23 @@ template <int GM, int DM, bool EXACT, int K, int WAVES>
 __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) void plan_in_one_launch(PlanArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ int rep_of_edge_all[kLpsPerWorkgroup * kWave];
-  __shared__ int flags[4];   // [0] the exchange of counts worked, [1] some share will not come,
-                             // [2] a wait of this workgroup ran out, [3] feasible LPs of this workgroup
+  __shared__ int flags[2];   // [0] the exchange of counts worked, [1] some share will not come
   const int nl = a.sh.n_logical, R = a.n_rep;
   const int tid = threadIdx.x;
   constexpr int nt = WAVES * kWave;
   const int lane = tid % kWave;
   const int wave_s = __builtin_amdgcn_readfirstlane(tid / kWave);   // wave-uniform
   const int pid = blockIdx.x;
-  const int n_shares = a.sh.n_ranks * a.sh.D;
+  // Which launch of this block of counters this is (the same value in every workgroup: it
+  // is advanced only once all of them have read it), and whether the block is switched off.
+  const int gen = agent_load(a.sync + kGenAt);
+  const bool poisoned = agent_load(a.sync + kPoisonAt) != 0;
+  const int parity = gen & 1;
+  const uint32_t tag_valid = (((uint32_t)gen + 1u) << 2) | 1u, tag_none = tag_valid + 1u;
+  int *arrived_stripes = a.sync + kArrivedAt + parity * kArrivalStripes;
   unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
-  unsigned long long *totals_acc = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt);   // [n_copies][nl]
+  unsigned long long *totals_acc =
+      reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + (size_t)parity * kTotalsWords;   // [n_copies][nl]
   // The batch's tokens of expert e and the number of slices that have contributed: the copies
   // added up (all loads in flight together); complete once every slice has arrived.
   auto batch_totals = [&](int e, int32_t &tokens, int32_t &slices) {
@@ -217,12 +173,15 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     // slices, fetches the totals the slices have added up in memory and hands them over.
     __shared__ int counts_ready;
     float *staged = reinterpret_cast<float *>(smem_raw);
-    if (tid == 0) {
+    if (tid == 0)
       counts_ready = 0;
-      flags[2] = 0;
-      flags[3] = 0;
-    }
     __syncthreads();
+    // This workgroup has read the launch counter: the first slice may advance it once
+    // every workgroup has said so.  (The last wave says it: the LP waves do not wait for
+    // the counter to arrive before they start.)
+    if (tid == nt - 1)
+      announce_arrival(arrived_stripes, a.n_slices + pid);
+    sa.tag_valid = tag_valid;
     if (a.local_counts) {
       sa.counts_ready = &counts_ready;
       if (wave_s == n_lps) {
@@ -242,10 +201,8 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
           if (!complete)
             __builtin_amdgcn_s_sleep(2);
         }
-        if (!complete && lane == 0) {
+        if (!complete && lane == 0)
           give_up(a);
-          flags[2] = 1;
-        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
           __hip_atomic_store(&counts_ready, complete ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -260,13 +217,12 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
         // no counts, no solution: tell the slices not to wait for this LP's shares
         const int n_edges = sa.G * sa.D;
         for (int j = lane; j < n_edges; j += kWave)
-          agent_store(shares + (int64_t)(first_lp + wave_s) * n_edges + j, 2ull << 32);
-      } else if (lane == 0 && n_ok > 0) {
-        atomicAdd(&flags[3], n_ok);
+          agent_store(shares + (int64_t)(first_lp + wave_s) * n_edges + j, (unsigned long long)tag_none << 32);
+      } else if (lane == 0 && n_ok > 0 && !poisoned) {
+        atomicAdd(a.avail, n_ok);
       }
     }
     LPLB_PLAN_STAMP(2);
-    leave(a, n_shares, &flags[2], &flags[3]);
     return;
   }
 
@@ -303,6 +259,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     s.group_rank = s.ep_rank - (int)fast_div((uint32_t)s.ep_rank, a.magic_G) * a.sh.G;
     return s;
   };
+  const int dirty_words = min(agent_load(a.sync + kDirtyAt + (1 - parity)), kTotalsWords);
   const int e0 = min(tid, nl - 1);
   const int slot0 = slot_of(e0);
   const int le0 = a.phy2log[slot0];
@@ -346,7 +303,6 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     reps[R] = RepEntry{1, 0xffffffffu, INT32_MAX, -1};   // "no replica": every token stays
     flags[0] = 0;
     flags[1] = 0;
-    flags[3] = 0;
   }
   __syncthreads();
   if (tid < nl && le0 >= 0 && le0 < nl)
@@ -370,6 +326,21 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   for (int i = tid + nt; i < R; i += nt) {
     const SetOf s = set_of(i);
     enter_set(i, s, a.phy2log[s.ep_rank * a.sh.P + s.place], a.o2r[s.group_rank * a.sh.D + s.d]);
+  }
+  // ---- housekeeping while the indices are on their way: the set of counters that the
+  // launch before this one used (nobody looks at it during this launch) is cleared for the
+  // launch after this one, every slice taking its part; the stores only have to be done
+  // when the kernel ends ----
+  if (!poisoned) {
+    unsigned long long *stale = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + (size_t)(1 - parity) * kTotalsWords;
+    for (int i = slice * nt + tid; i < dirty_words; i += a.n_slices * nt)
+      agent_store(stale + i, 0ull);
+    if (slice == 0) {
+      if (tid < kArrivalStripes)
+        agent_store(a.sync + kArrivedAt + (1 - parity) * kArrivalStripes + tid, 0);
+      if (tid == 0)
+        agent_store(a.sync + kDirtyAt + parity, a.n_copies * nl);
+    }
   }
   __syncthreads();
 
@@ -426,26 +397,35 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   __syncthreads();
   // ---- this slice's counts, for every workgroup: the histogram goes into the batch's
   // totals, the counts of the replicated sets into this slice's row ----
-  for (int e = tid; e < nl; e += nt) {
-    const int32_t mine = hist[e];
-    if (a.local_counts || mine != 0)   // (only the LP's poller looks at the number of contributions)
-      agent_add(totals_acc + (slice & (a.n_copies - 1)) * nl + e, ((unsigned long long)(uint32_t)mine << 32) | 1ull);
+  if (!poisoned) {
+    for (int e = tid; e < nl; e += nt) {
+      const int32_t mine = hist[e];
+      if (a.local_counts || mine != 0)   // (only the LP's poller looks at the number of contributions)
+        agent_add(totals_acc + (slice & (a.n_copies - 1)) * nl + e, ((unsigned long long)(uint32_t)mine << 32) | 1ull);
+    }
+    for (int q = tid; q < R; q += nt) {
+      const int le = set_expert[q];
+      agent_store(a.rows + (((int64_t)slice) << a.row_shift) + q, le >= 0 ? hist[le] : 0);
+    }
+    stores_have_landed();
   }
-  for (int q = tid; q < R; q += nt) {
-    const int le = set_expert[q];
-    agent_store(a.rows + (((int64_t)slice) << a.row_shift) + q, le >= 0 ? hist[le] : 0);
-  }
-  stores_have_landed();
   __syncthreads();
   LPLB_PLAN_STAMP(1);
   if (wave_s == 0) {
-    if (lane == 0)
-      announce_arrival(a.sync + kArrivedAt, slice);
-    const bool arrived = wait_for_arrivals(a.sync + kArrivedAt, a.expected_slices, a.max_polls);
-    if (lane == 0) {
-      if (!arrived)
-        give_up(a);
-      flags[0] = arrived;
+    if (poisoned) {
+      if (slice == 0 && lane == 0)
+        agent_add(a.sync + kTimeoutsAt, 1);   // one more plan that this block of counters could not serve
+    } else {
+      if (lane == 0)
+        announce_arrival(arrived_stripes, slice);
+      const bool arrived = wait_for_arrivals(arrived_stripes, a.expected_slices + a.n_lp_workgroups, a.max_polls);
+      if (lane == 0) {
+        if (!arrived)
+          give_up(a);
+        else if (slice == 0)
+          agent_store(a.sync + kGenAt, (gen + 1) & 0x3fffffff);   // every workgroup has read it by now
+        flags[0] = arrived;
+      }
     }
   }
   __syncthreads();
@@ -534,12 +514,14 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       const SetOf s = set_of(i);
       unsigned long long word = 0;
       int polls = 0;
-      while ((word = agent_load(shares + s.ep_rank * a.sh.D + s.d)) == 0 && ++polls < a.max_polls)
+      uint32_t tag = 0;
+      while ((tag = (uint32_t)((word = agent_load(shares + s.ep_rank * a.sh.D + s.d)) >> 32)) != tag_valid &&
+             tag != tag_none && ++polls < a.max_polls)
         __builtin_amdgcn_s_sleep(2);
-      if ((uint32_t)(word >> 32) == 1u) {
+      if (tag == tag_valid) {
         reps[R - 1 - i].expected = expected_on_original(__builtin_bit_cast(float, (uint32_t)word), total[R - 1 - i]);
       } else {
-        if (word == 0)
+        if (tag != tag_none)
           give_up(a);
         flags[1] = 1;
       }
@@ -565,14 +547,11 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       }
       a.physical_counts[i] = v;
     }
-    stores_have_landed();   // (a launch that gave up overwrites them from the last workgroup to leave)
   }
-  // This workgroup needs nothing from the others any more: it counts as gone now, so that the
-  // counters are cleared while the outputs are still being stored, not after them.
+  if (slice == 0 && a.physical_counts && !ok)
+    for (int i = tid; i < a.sh.n_ranks * a.sh.P; i += nt)
+      a.physical_counts[i] = -1;
   LPLB_PLAN_STAMP(6);
-  if (tid == 0)
-    flags[2] = !ok;
-  leave(a, n_shares, &flags[2], &flags[3]);
   // ---- choose and store; if a wait ran out, every token goes to its original slot ----
   {
     int64_t *dst = a.out + w0 + lane;
@@ -907,12 +886,23 @@ extern "C" int lplb_plan_sync_timeouts(int *count) {
   const int rc = plan_device(&d);
   if (rc != LPLB_OK)
     return rc;
+  // Everything enqueued so far has ended after this, so a block that is switched off can be
+  // cleared without a launch looking at it (the caller must not enqueue plans from other
+  // threads meanwhile, as the header says).
+  LPLB_HIP_TRY(hipDeviceSynchronize());
   *count = 0;
   for (int slot = 0; slot < kSyncSlots; ++slot) {
-    int n = 0;
-    LPLB_HIP_TRY(hipMemcpy(&n, d->sync + (size_t)slot * kSlotInts + kTimeoutsAt, sizeof(int), hipMemcpyDeviceToHost));
-    *count += n;
+    int *block = d->sync + (size_t)slot * kSlotInts;
+    int head[kTimeoutsAt + 1] = {};
+    LPLB_HIP_TRY(hipMemcpy(head, block, sizeof(head), hipMemcpyDeviceToHost));
+    *count += head[kTimeoutsAt];
+    if (head[kPoisonAt] != 0) {
+      // back to the state of a block that has never been used; the failures stay counted
+      LPLB_HIP_TRY(hipMemset(block, 0, kTimeoutsAt * sizeof(int)));
+      LPLB_HIP_TRY(hipMemset(block + kTimeoutsAt + 1, 0, (size_t)(kSlotInts - kTimeoutsAt - 1) * sizeof(int)));
+    }
   }
+  LPLB_HIP_TRY(hipDeviceSynchronize());
   return LPLB_OK;
 }
 

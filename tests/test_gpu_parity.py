@@ -1077,10 +1077,11 @@ def test_plan_at_the_sweep_shape_is_one_launch_and_equals_the_chain(cuda, use_gl
 def test_one_launch_plan_gives_up_in_a_defined_way(cuda, use_global):
     """A wait between workgroups that cannot be met (forced from the host: the kernel is told to expect
     one slice more than its grid has, and to poll 2000 times instead of millions) must end in the
-    documented fallback -- every token on its expert's original slot, the feasible-LP counter untouched,
-    physical_counts filled with -1, the give-ups counted -- with every kernel ending normally, and
-    the next plan on the same stream must be right again (minilp.cu:395-397 is the reference's own
-    neutral fallback for an LP that fails)."""
+    documented fallback -- every token on its expert's original slot, physical_counts filled with -1,
+    the give-ups counted -- with every kernel ending normally.  The block of counters the launch used
+    is switched off after that: the next plan on the stream falls back in the same way and counts one
+    more failure, until lplb_plan_sync_timeouts has been called; then plans are right again
+    (minilp.cu:395-397 is the reference's own neutral fallback for an LP that fails)."""
     from lplb_amd import _native
     inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
     lib = _native.load()
@@ -1095,28 +1096,33 @@ def test_one_launch_plan_gives_up_in_a_defined_way(cuda, use_global):
     timeouts_before, launches_before = _native.plan_sync_timeouts(), _native.plan_one_launch_count()
     print("injecting a wait that cannot be met", flush=True)
     assert lib.lplb_plan_inject_fault(1, 2000) == 0
-    out, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
-                            physical_counts=phys)
-    torch.cuda.synchronize()
-    assert _native.plan_one_launch_count() == launches_before + 1
     # the fallback: the redirect with every share = 1 keeps every token on the original
     by_sm = oracle.count_idx(inp.indices, shape.n_logical, 256)
     stay = oracle.map_idx(inp.indices, np.ones((1, shape.G, shape.D), np.float32), by_sm, shape.o2r, inp.phy2log, 1,
                           shape.C, shape.P)
-    np.testing.assert_array_equal(out.cpu().numpy(), stay)
-    assert int(avail[0]) == 1                       # withheld
-    assert torch.all(phys == -1)
-    gave_up = _native.plan_sync_timeouts() - timeouts_before
-    assert gave_up >= 64, gave_up                   # every slice workgroup's wait (and the LP's, if it waited too)
+    for later in range(2):   # the launch in which the wait runs out, then one that finds the block switched off
+        phys.fill_(-7)
+        out, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
+                                physical_counts=phys)
+        torch.cuda.synchronize()
+        assert _native.plan_one_launch_count() == launches_before + 1 + later
+        np.testing.assert_array_equal(out.cpu().numpy(), stay)
+        assert torch.all(phys == -1)
+    # (with the counts supplied the LP needs nothing from the slices and is solved all the same in the
+    # first of the two launches; a launch that finds the block switched off adds nothing)
+    assert int(avail[0]) == (2 if use_global else 1)
+    gave_up = _native.plan_sync_timeouts() - timeouts_before      # ... which also switches the block on again
+    assert gave_up >= 64 + 1, gave_up           # every slice workgroup's wait (and the LP's, if it waited too), and the second plan
     # the next plans on the same stream are healthy
+    avail.zero_()
     for _ in range(3):
         out, o_w, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=counts,
                                   physical_counts=phys)
         torch.cuda.synchronize()
         assert torch.equal(out, want) and torch.equal(o_w, want_w) and torch.equal(phys, want_phys)
-    assert int(avail[0]) == 4
+    assert int(avail[0]) == 3
     assert _native.plan_sync_timeouts() - timeouts_before == gave_up
-    assert _native.plan_one_launch_count() == launches_before + 4
+    assert _native.plan_one_launch_count() == launches_before + 5
 
 
 def test_one_launch_slots_pass_from_stream_to_stream(cuda):
