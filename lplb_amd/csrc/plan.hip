@@ -153,7 +153,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     unsigned long long v[kTotalCopies];
 #pragma unroll
     for (int k = 0; k < kTotalCopies; ++k)
-      v[k] = totals_acc[(k & (a.n_copies - 1)) * nl + e];
+      v[k] = agent_load(totals_acc + (k & (a.n_copies - 1)) * nl + e);
     unsigned long long sum = 0;
 #pragma unroll
     for (int k = 0; k < kTotalCopies; ++k)
@@ -186,10 +186,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       sa.counts_ready = &counts_ready;
       if (wave_s == n_lps) {
         // Poll the batch's totals until every expert's words say that all slices have
-        // added theirs (plain loads after an acquire: they can be batched).
+        // added theirs.
         bool complete = false;
         for (int polls = 0; polls < a.max_polls && !complete; ++polls) {
-          see_other_workgroups();
           bool all_in = true;
           for (int e = lane; e < nl; e += kWave) {
             int32_t tokens, slices;
@@ -259,7 +258,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     s.group_rank = s.ep_rank - (int)fast_div((uint32_t)s.ep_rank, a.magic_G) * a.sh.G;
     return s;
   };
-  const int dirty_words = min(agent_load(a.sync + kDirtyAt + (1 - parity)), kTotalsWords);
+  const int dirty0 = agent_load(a.sync + kDirtyAt), dirty1 = agent_load(a.sync + kDirtyAt + 1);
   const int e0 = min(tid, nl - 1);
   const int slot0 = slot_of(e0);
   const int le0 = a.phy2log[slot0];
@@ -332,6 +331,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   // launch after this one, every slice taking its part; the stores only have to be done
   // when the kernel ends ----
   if (!poisoned) {
+    const int dirty_words = min(parity ? dirty0 : dirty1, kTotalsWords);   // of the set with the other parity
     unsigned long long *stale = reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + (size_t)(1 - parity) * kTotalsWords;
     for (int i = slice * nt + tid; i < dirty_words; i += a.n_slices * nt)
       agent_store(stale + i, 0ull);
@@ -343,6 +343,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     }
   }
   __syncthreads();
+  LPLB_PLAN_STAMP(10);
 
   // ---- the tokens: histogram of the slice, bitmaps of the replicated sets per chunk ----
   // Between the phases a token is kept as its expert id only, two ids per register (the
@@ -367,6 +368,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       atomicAdd(&hist[e], 1);
   }
   __syncthreads();
+  LPLB_PLAN_STAMP(8);
   // ---- inside the wave: tokens of each set in the chunks before each chunk (lane = (set,
   // chunk), chunk fastest), and in all of the wave's chunks ----
   if (R > 0) {
@@ -397,6 +399,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   __syncthreads();
   // ---- this slice's counts, for every workgroup: the histogram goes into the batch's
   // totals, the counts of the replicated sets into this slice's row ----
+  LPLB_PLAN_STAMP(9);
   if (!poisoned) {
     for (int e = tid; e < nl; e += nt) {
       const int32_t mine = hist[e];
@@ -431,10 +434,21 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   __syncthreads();
   LPLB_PLAN_STAMP(2);
   bool ok = flags[0] != 0;   // (the same in every thread)
-  int32_t h[K];
+  // Hashes of this thread's tokens: worked out while the LP is still running where a
+  // thread has few tokens (short batches, where the LP is the longest chain); with many
+  // tokens per thread they are worked out at the end, one token at a time, which keeps the
+  // kernel inside the registers that let two workgroups share a CU.
+  constexpr bool kHashEarly = K <= 4;
+  int32_t h[kHashEarly ? K : 1];
+  auto hash_of_chunk = [&](int c) {
+    const int set = route[expert_of_chunk(c)].rep;
+    const i32x4 s = *reinterpret_cast<const i32x4 *>(slot_of_chunk(set, c));   // bits_lo, bits_hi, start
+    const i32x4 x = *reinterpret_cast<const i32x4 *>(&reps[set]);              // total, magic, -, -
+    const int32_t k =
+        __builtin_amdgcn_mbcnt_hi((uint32_t)s.y, __builtin_amdgcn_mbcnt_lo((uint32_t)s.x, (uint32_t)s.z));
+    return ordinal_hash<false>(k, x.x, (uint32_t)x.y);
+  };
   if (ok) {
-    // (wave 0's wait ended with the acquire that lets the plain loads below see the other
-    // workgroups' rows: one invalidate per workgroup, not one per wave)
     // ---- tokens of each replicated set before this slice and in the whole batch: a thread
     // takes one set of every (threads / row length)-th slice, loads in batches ----
     {
@@ -448,7 +462,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
           int32_t v[kInFlight];
 #pragma unroll
           for (int k = 0; k < kInFlight; ++k)
-            v[k] = a.rows[(((int64_t)min(p0 + k * p_lanes, a.n_slices - 1)) << a.row_shift) + q];
+            v[k] = agent_load(a.rows + ((((int64_t)min(p0 + k * p_lanes, a.n_slices - 1)) << a.row_shift) + q));
 #pragma unroll
           for (int k = 0; k < kInFlight; ++k) {
             const int p = p0 + k * p_lanes;
@@ -456,8 +470,15 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
             b_sum += p < slice ? v[k] : 0;
           }
         }
-        atomicAdd(&total[q], t_sum);
-        atomicAdd(&before[q], b_sum);
+        // lanes of a wave that hold the same set add up first (updates of one LDS word queue up)
+        for (int m = q_lanes; m < kWave; m <<= 1) {
+          t_sum += __shfl_xor(t_sum, m);
+          b_sum += __shfl_xor(b_sum, m);
+        }
+        if (lane < q_lanes) {
+          atomicAdd(&total[q], t_sum);
+          atomicAdd(&before[q], b_sum);
+        }
       }
     }
     if (slice == 0)   // this GPU's tokens per expert, for the caller (and for the counts below)
@@ -499,14 +520,10 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     __syncthreads();
     LPLB_PLAN_STAMP(4);
     // ---- ordinals and hashes of the tokens, while the LP is still running ----
+    if constexpr (kHashEarly) {
 #pragma unroll
-    for (int c = 0; c < K; ++c) {
-      const int set = route[expert_of_chunk(c)].rep;
-      const i32x4 s = *reinterpret_cast<const i32x4 *>(slot_of_chunk(set, c));   // bits_lo, bits_hi, start
-      const i32x4 x = *reinterpret_cast<const i32x4 *>(&reps[set]);              // total, magic, -, -
-      const int32_t k =
-          __builtin_amdgcn_mbcnt_hi((uint32_t)s.y, __builtin_amdgcn_mbcnt_lo((uint32_t)s.x, (uint32_t)s.z));
-      h[c] = ordinal_hash<false>(k, x.x, (uint32_t)x.y);
+      for (int c = 0; c < K; ++c)
+        h[c] = hash_of_chunk(c);
     }
     // ---- the LP's shares: every set's thread polls its own; value and tag arrive in
     // the same 8-byte word ----
@@ -562,7 +579,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       o[c] = rt.original;
       if (ok) {
         const RepEntry x = reps[rt.rep];
-        o[c] = h[c] >= x.expected ? x.replica : rt.original;
+        o[c] = (kHashEarly ? h[c] : hash_of_chunk(c)) >= x.expected ? x.replica : rt.original;
       }
     }
     if (whole) {

@@ -10,8 +10,9 @@
 //   * s_waitcnt vmcnt(0) after such stores waits for their acknowledgement, i.e. until
 //     they are visible device-wide; the counter that announces them is bumped only
 //     after that wait and a workgroup barrier;
-//   * an agent-scope acquire fence (buffer_inv sc1) makes the plain loads that follow it
-//     miss in this CU's L1 and this XCD's L2, so they can be ordinary, batched loads;
+//   * everything a workgroup reads of another's is read with such loads, never with plain
+//     loads behind an acquire fence: the fence (buffer_inv sc1) would invalidate this XCD's
+//     L2, which holds the batch's indices at that point, once per workgroup;
 //   * the compiler does not move memory operations across s_waitcnt / fences / atomics
 //     of the same or wider scope.
 // tests/test_host.py compiles these helpers on their own and checks that the sc1 forms
@@ -43,8 +44,6 @@ __device__ inline void agent_add(unsigned long long *p, unsigned long long v) {
 }
 // All earlier stores and atomics of this wave have been acknowledged.
 __device__ inline void stores_have_landed() { __builtin_amdgcn_s_waitcnt(0); }
-// Plain loads after this see what other workgroups wrote through before they signalled.
-__device__ inline void see_other_workgroups() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
 
 // Counting arrivals.  Updates of one address queue up behind each other (about 35 ns
 // each), so a counter that hundreds of workgroups bump would itself take microseconds;
@@ -54,6 +53,8 @@ constexpr int kArrivalStripes = 16;
 __device__ inline void announce_arrival(int *stripes, int id) { agent_add(stripes + id % kArrivalStripes, 1); }
 // All 64 lanes of one wave poll the stripes until they add up to `target` or `max_polls`
 // polls have passed.  Returns whether the target was reached (the same in every lane).
+// What the arrived workgroups wrote before they announced themselves is in memory then;
+// read it with agent_load.
 __device__ inline bool wait_for_arrivals(int *stripes, int target, int max_polls) {
   const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   bool reached = false;
@@ -66,7 +67,6 @@ __device__ inline bool wait_for_arrivals(int *stripes, int target, int max_polls
     if (!reached)
       __builtin_amdgcn_s_sleep(2);
   }
-  see_other_workgroups();
   return reached;
 }
 
