@@ -56,7 +56,8 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   [kPoisonAt] non-zero: a wait ran out in this block (see above); [kTimeoutsAt] waits that
 //   ran out since the library was loaded (never cleared);
 //   [kDirtyAt + p] how many words of set p's totals the last launch that used it may have left non-zero;
-//   [kArrivedAt + 16 p ..] workgroups that have published (slices) or started (LP), striped;
+//   from kArrivedAt: workgroups that have published (slices) or started (LP): per set p,
+//   kArrivalCopies copies of a striped counter (plan_sync.h);
 //   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits with
 //   tag = (launch tag << 2) | 1 (valid) or 2 (there will be none); a word with another
 //   launch's tag is "not there yet";
@@ -67,12 +68,13 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   updates of one address queue up behind each other, about 35 ns each, so one copy per 16
 //   slices (at most kTotalCopies); whoever needs the batch's tokens per expert adds the copies up.
 constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8;
-constexpr int kArrivedAt = 16;      // 2 x kArrivalStripes words, a 64-byte line each
-constexpr int kSharesAt = 48, kMaxShares = 1024;
+constexpr int kSharesAt = 16, kMaxShares = 1024;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024, kTotalCopies = 16;
 constexpr int kTotalsWords = kTotalCopies * kMaxTotals;   // 8-byte words of one set
-constexpr int kSlotInts = kTotalsAt + 2 * 2 * kTotalsWords, kSyncSlots = 8;
-static __device__ __attribute__((aligned(64))) int g_plan_sync[kSyncSlots * kSlotInts];
+constexpr int kArrivedAt = kTotalsAt + 2 * 2 * kTotalsWords;   // [2][kArrivalCopies][kArrivalCopyInts]
+constexpr int kSlotInts = kArrivedAt + 2 * kArrivalCopies * kArrivalCopyInts, kSyncSlots = 8;
+static_assert(kArrivedAt % 16 == 0 && kSlotInts % 16 == 0, "the counters' lines are 64-byte aligned");
+static __device__ __attribute__((aligned(4096))) int g_plan_sync[kSyncSlots * kSlotInts];
 static std::atomic<bool> g_cooperative{true};   // any thread may flip it while others plan
 static std::atomic<long long> g_one_launch_plans{0};
 // Test hook (lplb_plan_inject_fault): the next one-launch plan expects this many slices
@@ -84,6 +86,7 @@ struct PlanArgs {
   int64_t n, per;
   int n_slices, n_lp_workgroups;
   int n_copies;          // partial histograms of the batch: a power of two, at most kTotalCopies
+  int n_arrival_copies;  // copies of the arrival counter: a power of two, at most kArrivalCopies
   int expected_slices;   // = n_slices unless a fault is injected
   int max_polls;
   const int32_t *o2r, *phy2log;
@@ -122,6 +125,17 @@ static size_t plan_lds_bytes(int n_logical, int n_rep, int n_waves, int k) {
                 : blockIdx.x == gridDim.x - 1 ? a.solve.clocks + 80                            \
                 : blockIdx.x == 0 ? a.solve.clocks + 96 : nullptr, k)
 
+// Debug builds: stamps of every slice workgroup (the buffer must hold 128 + 8 * slices).
+#ifdef LPLB_PHASE_CLOCKS
+#define LPLB_SLICE_STAMP(k)                                                                    \
+  do {                                                                                         \
+    if (a.solve.clocks && threadIdx.x == 0)                                                    \
+      a.solve.clocks[128 + 8 * (blockIdx.x - a.n_lp_workgroups) + (k)] = wall_clock64();       \
+  } while (0)
+#else
+#define LPLB_SLICE_STAMP(k) do { } while (0)
+#endif
+
 // K: 64-index chunks per wave.  WAVES: waves per workgroup.
 // Registers: with LP shapes that fit 128 VGPRs the kernel as a whole is held to 128 (four
 // waves per SIMD: one 16-wave or two 8-wave workgroups per CU), which is what lets the 257
@@ -143,7 +157,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   const bool poisoned = agent_load(a.sync + kPoisonAt) != 0;
   const int parity = gen & 1;
   const uint32_t tag_valid = (((uint32_t)gen + 1u) << 2) | 1u, tag_none = tag_valid + 1u;
-  int *arrived_stripes = a.sync + kArrivedAt + parity * kArrivalStripes;
+  int *arrived_stripes = a.sync + kArrivedAt + parity * (kArrivalCopies * kArrivalCopyInts);
   unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
   unsigned long long *totals_acc =
       reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + (size_t)parity * kTotalsWords;   // [n_copies][nl]
@@ -179,8 +193,8 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     // This workgroup has read the launch counter: the first slice may advance it once
     // every workgroup has said so.  (The last wave says it: the LP waves do not wait for
     // the counter to arrive before they start.)
-    if (tid == nt - 1)
-      announce_arrival(arrived_stripes, a.n_slices + pid);
+    if (wave_s == WAVES - 1)
+      announce_arrival(arrived_stripes, a.n_arrival_copies, a.n_slices + pid);
     sa.tag_valid = tag_valid;
     if (a.local_counts) {
       sa.counts_ready = &counts_ready;
@@ -236,13 +250,19 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   int32_t *set_expert = hist + nl;                                                  // [R]
   int32_t *before = set_expert + R;                                                 // [R] tokens of the set before this slice
   int32_t *total = before + R;                                                      // [R] ... in the whole batch
-  int32_t *wave_total = total + R;                                                  // [WAVES][R] ... in each wave's chunks
+  int32_t *wave_total = total + R;                                                  // [WAVES][R] ... in each wave's chunks, then in the chunks of the waves before it
   unsigned char *my_records = records + (size_t)wave_s * wave_stride;
   const unsigned long long my_bit = 1ull << lane;
   const int64_t begin = slice_begin(a.n, a.per, slice);
   const int64_t end = slice_begin(a.n, a.per, slice + 1);
   const int cd = a.sh.C * a.sh.D;
   LPLB_PLAN_STAMP(0);
+  LPLB_SLICE_STAMP(0);
+  // Where a slice shares a CU with an LP workgroup (grids with more workgroups than CUs), its
+  // waves go first: the LP wave issues an instruction nearly every cycle it may, and a slice
+  // wave on the same SIMD would be starved for as long as the LP runs, with every other slice
+  // waiting for it.  The slices spend most of their time asleep, so the LP loses little.
+  __builtin_amdgcn_s_setprio(2);
 
   // ---- small table reads first (they need no counts), then the index loads; all of
   // them unconditional loads from clamped addresses, so that nothing waits here ----
@@ -336,8 +356,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     for (int i = slice * nt + tid; i < dirty_words; i += a.n_slices * nt)
       agent_store(stale + i, 0ull);
     if (slice == 0) {
-      if (tid < kArrivalStripes)
-        agent_store(a.sync + kArrivedAt + (1 - parity) * kArrivalStripes + tid, 0);
+      if (tid < kArrivalCopies * kArrivalStripes)
+        agent_store(a.sync + kArrivedAt + ((1 - parity) * kArrivalCopies + tid / kArrivalStripes) * kArrivalCopyInts +
+                        (tid % kArrivalStripes) * kArrivalStripeInts, 0);
       if (tid == 0)
         agent_store(a.sync + kDirtyAt + parity, a.n_copies * nl);
     }
@@ -369,6 +390,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   }
   __syncthreads();
   LPLB_PLAN_STAMP(8);
+  LPLB_SLICE_STAMP(1);
   // ---- inside the wave: tokens of each set in the chunks before each chunk (lane = (set,
   // chunk), chunk fastest), and in all of the wave's chunks ----
   if (R > 0) {
@@ -390,8 +412,11 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   __syncthreads();
   for (int q = tid; q < R; q += nt) {   // the sets' tokens in this slice, into the histogram
     int32_t n = 0;
-    for (int w = 0; w < WAVES; ++w)
-      n += wave_total[w * R + q];
+    for (int w = 0; w < WAVES; ++w) {   // (and each wave's count becomes the count of the waves before it)
+      const int32_t of_wave = wave_total[w * R + q];
+      wave_total[w * R + q] = n;
+      n += of_wave;
+    }
     const int le = set_expert[q];
     if (le >= 0 && route[le].rep == q)   // (of two sets that name the same expert only one has the tokens)
       hist[le] = n;
@@ -414,14 +439,15 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   }
   __syncthreads();
   LPLB_PLAN_STAMP(1);
+  LPLB_SLICE_STAMP(2);
   if (wave_s == 0) {
     if (poisoned) {
       if (slice == 0 && lane == 0)
         agent_add(a.sync + kTimeoutsAt, 1);   // one more plan that this block of counters could not serve
     } else {
-      if (lane == 0)
-        announce_arrival(arrived_stripes, slice);
-      const bool arrived = wait_for_arrivals(arrived_stripes, a.expected_slices + a.n_lp_workgroups, a.max_polls);
+      announce_arrival(arrived_stripes, a.n_arrival_copies, slice);
+      const bool arrived = wait_for_arrivals(arrived_stripes + (slice & (a.n_arrival_copies - 1)) * kArrivalCopyInts,
+                                             a.expected_slices + a.n_lp_workgroups, a.max_polls);
       if (lane == 0) {
         if (!arrived)
           give_up(a);
@@ -433,6 +459,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   }
   __syncthreads();
   LPLB_PLAN_STAMP(2);
+  LPLB_SLICE_STAMP(4);
   bool ok = flags[0] != 0;   // (the same in every thread)
   // Hashes of this thread's tokens: worked out while the LP is still running where a
   // thread has few tokens (short batches, where the LP is the longest chain); with many
@@ -503,16 +530,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
       for (int p0 = 0; p0 < R * K; p0 += kWave) {
         const bool live = p0 + lane < R * K;
         const int q = live ? (p0 + lane) / K : 0;
-        int32_t base = before[q];
-        for (int v0 = 0; v0 < wave_s; v0 += 4) {
-          int32_t t[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            t[u] = wave_total[min(v0 + u, wave_s) * R + q];
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            base += v0 + u < wave_s ? t[u] : 0;
-        }
+        const int32_t base = before[q] + wave_total[wave_s * R + q];
         if (live)
           atomicAdd(&(reinterpret_cast<ChunkSlot *>(my_records + __umul24((uint32_t)q, (uint32_t)kRec)) + c)->start, base);
       }
@@ -594,6 +612,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     }
   }
   LPLB_PLAN_STAMP(7);
+  LPLB_SLICE_STAMP(3);
 }
 
 // LP shapes the one-launch plan is built for, in the order they are tried, and the
@@ -870,6 +889,9 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   a.n_copies = 1;
   while (a.n_copies < kTotalCopies && a.n_copies * 16 < a.n_slices)
     a.n_copies *= 2;
+  a.n_arrival_copies = 1;
+  while (a.n_arrival_copies < kArrivalCopies && a.n_arrival_copies * 32 < a.n_slices)
+    a.n_arrival_copies *= 2;
   SolveArgs &sa = a.solve;
   sa.workload = counts; sa.gw_out = global_workload; sa.r2o = r2o; sa.phy2log = phy2log;
   sa.avail = avail_num; sa.result = o_weight; sa.n_group = n_group; sa.G = G; sa.D = D; sa.C = C;

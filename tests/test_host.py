@@ -244,8 +244,8 @@ extern "C" __global__ void publish(int *row, unsigned long long *word, int *coun
   agent_add(word, (5ull << 32) | 1ull);
   stores_have_landed();
   __syncthreads();
-  if (threadIdx.x == 0)
-    announce_arrival(counter, blockIdx.x);
+  if (threadIdx.x < 64)
+    announce_arrival(counter, 4, blockIdx.x);
 }
 extern "C" __global__ void consume(int *counter, const int *row, const unsigned long long *word, int *out) {
   if (threadIdx.x < 64)
