@@ -162,10 +162,12 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
 /*
  * One batch's whole plan in a single call: what Planner.run does with three
  * extension calls (lplb/planner.py:245-266), with the same results as
- * lplb_count_idx, lplb_solve and lplb_map_idx chained on `stream`.  Short
- * batches (up to 524288 indices) of LP shapes up to 32 x 2 and up to 32 EP groups run as ONE kernel launch in
- * which the workgroups exchange their histogram rows and the LP's result through
- * memory; everything else runs as the chain of the three entry points' kernels.
+ * lplb_count_idx, lplb_solve and lplb_map_idx chained on `stream`.  Batches of up
+ * to about two million indices (slices of at most 8192 indices, as many of them as
+ * fit the GPU together) with LP shapes up to 32 x 2, up to 32 EP groups and up to 1024
+ * logical experts run as ONE kernel launch in which the workgroups exchange their
+ * counts and the LP's result through memory; everything else runs as the chain of
+ * the three entry points' kernels.
  *
  *   global_counts    int32 [n_logical] or NULL.  NULL: the LP is fed this GPU's
  *                    own histogram, as Planner.run does without a process
@@ -182,17 +184,25 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
  *   physical_counts  int32 [n_physical] or NULL, out (see lplb_map_idx)
  *
  * The one-launch form: its workgroups wait for each other, so the whole grid has to be
- * resident on the GPU.  The library admits a launch only if the grid fits (occupancy
- * query) beside the one-launch plans that are still executing, of which it keeps
+ * resident on the GPU.  The library admits a launch only if the grid fits (worked out
+ * from the kernel's registers and LDS) beside the one-launch plans that are still executing, of which it keeps
  * track per stream (eight streams per device at a time; it asks the runtime whether
  * those streams still have work pending, it never waits); otherwise the call runs the
  * chain, with identical results.  A plan captured into a graph keeps its share of the GPU reserved
  * from then on (its replays are invisible to the library).  Launches on one stream never overlap; the exception the
  * library cannot see is a graph captured on one stream and replayed concurrently on
  * several (see lplb_plan_set_cooperative).  Every wait inside the kernel is bounded; if one
- * runs out (lplb_plan_sync_timeouts), the launch still completes with a valid but
- * unbalanced result: the tokens of the affected slices go to their experts' original
- * slots, avail_num is left unchanged and physical_counts, if given, is filled with -1.
+ * runs out, the launch still completes, with a valid but unbalanced result: the tokens of
+ * the slices whose wait ran out go to their experts' original slots (so every entry of
+ * `out` still names a slot that holds the token's expert).  The failure is counted
+ * (lplb_plan_sync_timeouts) and the caller has to look at that counter before it trusts
+ * what else the calls since its last look returned: physical_counts is filled with -1 when
+ * the workgroup that writes it is among those that gave up (always the case when the
+ * counts of the batch never became complete), the last row of counts_by_block may not have
+ * been written, avail_num counts the LPs that were solved, whether or not the slices got to
+ * use them.  After such a failure the stream's later plans that would run as one launch
+ * send every token to the original slot and count one more failure each, until
+ * lplb_plan_sync_timeouts has been called.
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -245,8 +255,10 @@ int lplb_plan_set_cooperative(int enabled);
  * No counterpart in the reference.  The workgroups of the one-launch plan wait
  * for each other with a bounded number of polls; *count receives how many waits
  * ran out on the current device since the library was loaded (0 in a healthy
- * run; what a plan with such a wait returns is described at lplb_plan).
- * Synchronous: copies a few ints from the device.
+ * run; what a plan with such a wait returns is described at lplb_plan), and the
+ * one-launch form is switched on again for the streams on which a wait had run out.
+ * Synchronous: waits for everything enqueued on the device, then copies a few ints.  Not
+ * to be called while a stream is being captured or while other threads enqueue plans.
  */
 int lplb_plan_sync_timeouts(int *count);
 

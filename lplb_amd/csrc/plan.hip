@@ -65,8 +65,9 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   words with the tokens in the high half and the number of slices that have contributed in
 //   the low half (one atomic add delivers both, so whoever polls the words needs no second
 //   round trip for a "done" counter).  Slice s adds its histogram to copy s % n_copies:
-//   updates of one address queue up behind each other, about 35 ns each, so one copy per 16
-//   slices (at most kTotalCopies); whoever needs the batch's tokens per expert adds the copies up.
+//   updates of one address queue up behind each other, so one copy per 16 slices (at most
+//   kTotalCopies; more copies cost whoever adds them up more than they save: measured);
+//   whoever needs the batch's tokens per expert adds the copies up.
 constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8;
 constexpr int kSharesAt = 16, kMaxShares = 1024;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024, kTotalCopies = 16;
@@ -411,11 +412,14 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
   }
   __syncthreads();
   for (int q = tid; q < R; q += nt) {   // the sets' tokens in this slice, into the histogram
-    int32_t n = 0;
-    for (int w = 0; w < WAVES; ++w) {   // (and each wave's count becomes the count of the waves before it)
-      const int32_t of_wave = wave_total[w * R + q];
+    int32_t n = 0, of_wave[WAVES];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      of_wave[w] = wave_total[w * R + q];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {   // (each wave's count becomes the count of the waves before it)
       wave_total[w * R + q] = n;
-      n += of_wave;
+      n += of_wave[w];
     }
     const int le = set_expert[q];
     if (le >= 0 && route[le].rep == q)   // (of two sets that name the same expert only one has the tokens)

@@ -270,3 +270,26 @@ extern "C" __global__ void consume(int *counter, const int *row, const unsigned 
     assert "s_sleep" in polls and re.search(r"global_load_dword .* sc1", polls), "a poll may hit a stale L2 line"
     assert re.search(r"global_load_dword v\d+, v\d+, s\[\d+:\d+\] sc1", after_wait), "the row is not read past the L2"
     assert re.search(r"global_load_dwordx2 .* sc1", after_wait), "the tagged word is read past the L2"
+
+
+def test_no_kernel_spills_vector_registers():
+    """The build leaves the compiler's per-kernel resource report next to each object
+    (lplb_amd/csrc/*.resources.txt).  No kernel may spill vector registers: besides being slow,
+    a spill placed where only part of a wave is active (seen with this compiler in a variant of the
+    one-launch plan, between a divergent loop and the instruction that restores the execution mask) loses
+    the value in the inactive lanes.  The variants are sized so that none spills; this keeps it so."""
+    reports = sorted((Path(__file__).parent.parent / "lplb_amd" / "csrc").glob("*.resources.txt"))
+    if not reports:
+        pytest.skip("no resource reports: the library was not built here")
+    n_kernels, spilling = 0, []
+    for report in reports:
+        name = None
+        for line in report.read_text().splitlines():
+            m = re.search(r"Function Name: (\S+)", line)
+            if m:
+                name, n_kernels = m.group(1), n_kernels + 1
+            m = re.search(r"VGPRs Spill: (\d+)", line)
+            if m and int(m.group(1)) > 0:
+                spilling.append((report.name, name, int(m.group(1))))
+    assert n_kernels > 100, n_kernels
+    assert not spilling, spilling
