@@ -124,8 +124,34 @@ def _stream(t: torch.Tensor) -> int:
 class CompiledSolver:
     """Launches the three planning kernels for one (n_group, G, D, P, C) shape."""
 
-    def __init__(self, n_group: int, group_size: int, dup_per_rank: int, n_local_experts: int,
-                 n_combined_experts: int) -> None:
+    def __init__(self, *args, **kwargs) -> None:
+        """Two ways to construct one.  The reference's own argument list (csrc/plugin.cpp:665-667,
+        as lplb/planner.py:26-35 passes it):
+            CompiledSolver(resource_path, n_group, group_size, dup_per_rank, block_dim,
+                           n_local_experts, n_combined_experts, pg)
+        where resource_path (the CUDA templates' folder) and block_dim (every kernel here picks its
+        own workgroup size) are accepted and ignored and pg is kept as .pg for the caller; or the
+        five numbers that matter:
+            CompiledSolver(n_group, group_size, dup_per_rank, n_local_experts, n_combined_experts)"""
+        self.pg = None
+        if args and isinstance(args[0], (str, bytes)) or "resource_path" in kwargs:
+            names = ("resource_path", "n_group", "group_size", "dup_per_rank", "block_dim", "n_local_experts",
+                     "n_combined_experts", "pg")
+        else:
+            names = ("n_group", "group_size", "dup_per_rank", "n_local_experts", "n_combined_experts")
+        if len(args) > len(names):
+            raise TypeError(f"CompiledSolver takes {len(names)} arguments {names}, got {len(args)}")
+        given = dict(zip(names, args))
+        for k, v in kwargs.items():
+            if k not in names or k in given:
+                raise TypeError(f"CompiledSolver: unexpected or repeated argument {k!r}")
+            given[k] = v
+        missing = [k for k in names if k not in given and k != "pg"]
+        if missing:
+            raise TypeError(f"CompiledSolver: missing arguments {missing}")
+        n_group, group_size, dup_per_rank = int(given["n_group"]), int(given["group_size"]), int(given["dup_per_rank"])
+        n_local_experts, n_combined_experts = int(given["n_local_experts"]), int(given["n_combined_experts"])
+        self.pg = given.get("pg")
         self.lib = load()
         self.n_group = n_group
         self.group_size = group_size

@@ -48,11 +48,16 @@ template <int GM, int DM, bool EXACT> static void launch_exactness(const SolveAr
   launch_variant<GM, DM, EXACT, 1>(a, s);
 }
 
+// A group that fills an instantiation exactly gets the variant whose loop bounds are all
+// compile-time constants.  Instantiations with more than 64 edges (16 x 8, 32 x 4) exist only
+// for the padded groups inside them (say 10 x 5 or 20 x 3): a group that filled them would
+// have more edges than a wave has lanes and has been refused by then.
 template <int GM, int DM> static void launch_solver(const SolveArgs &a, hipStream_t s) {
-  if (a.G == GM && a.D == DM)
-    launch_exactness<GM, DM, true>(a, s);
-  else
-    launch_exactness<GM, DM, false>(a, s);
+  if constexpr (GM * DM <= kWave) {
+    if (a.G == GM && a.D == DM)
+      return launch_exactness<GM, DM, true>(a, s);
+  }
+  launch_exactness<GM, DM, false>(a, s);
 }
 
 static int dispatch(const SolveArgs &a, hipStream_t s) {

@@ -293,3 +293,22 @@ def test_no_kernel_spills_vector_registers():
                 spilling.append((report.name, name, int(m.group(1))))
     assert n_kernels > 100, n_kernels
     assert not spilling, spilling
+
+
+def test_compiled_solver_takes_the_reference_argument_list():
+    """csrc/plugin.cpp:665-667 / lplb/planner.py:26-35: (resource_path, n_group, group_size, dup_per_rank,
+    block_dim, n_local_experts, n_combined_experts, pg)."""
+    from lplb_amd import _native
+    short = _native.CompiledSolver(2, 8, 2, 34, 1)
+    ref = _native.CompiledSolver("/somewhere/resources", 2, 8, 2, 256, 34, 1, None)
+    kw = _native.CompiledSolver(resource_path="x", n_group=2, group_size=8, dup_per_rank=2, block_dim=256,
+                                n_local_experts=34, n_combined_experts=1, pg="a group")
+    for s_ in (ref, kw):
+        assert (s_.n_group, s_.group_size, s_.dup_per_rank, s_.n_local_experts, s_.n_combined_experts, s_.n_experts) == \
+               (short.n_group, short.group_size, short.dup_per_rank, short.n_local_experts, short.n_combined_experts,
+                short.n_experts)
+    assert kw.pg == "a group" and ref.pg is None
+    with pytest.raises(TypeError):
+        _native.CompiledSolver("/somewhere/resources", 2, 8, 2, 256, 34)
+    with pytest.raises(TypeError):
+        _native.CompiledSolver(2, 8, 2, 34, 1, None)
