@@ -224,12 +224,19 @@ class CompiledSolver:
         return (result, gw) if want_global else result
 
     # -- csrc/plugin.cpp:580-600 -------------------------------------------------
-    def count_idx(self, idx: torch.Tensor, n_sms: int, block_dim: int = 256) -> tuple[torch.Tensor, torch.Tensor]:
+    def count_idx(self, idx: torch.Tensor, n_sms: int, block_dim: int = 256, *,
+                  out: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """out: optional int32 [n_sms, n_experts] table to fill instead of a new one (no counterpart in the
+        reference, which allocates on every call)."""
         _require(idx.dtype == torch.int64, "idx.dtype == int64")
         _require(idx.is_cuda, "idx.device().is_cuda()")
         _require(idx.is_contiguous(), "idx.is_contiguous()")
         _require(block_dim == 256, "slices are aligned to 256 indices")
-        out = torch.empty((n_sms, self.n_experts), dtype=torch.int32, device=idx.device)
+        if out is None:
+            out = torch.empty((n_sms, self.n_experts), dtype=torch.int32, device=idx.device)
+        else:
+            _require(out.dtype == torch.int32 and out.is_cuda and out.is_contiguous() and
+                     tuple(out.shape) == (n_sms, self.n_experts), "out: int32 [n_sms, n_experts], contiguous, on the GPU")
         _check(self.lib.lplb_count_idx(idx.data_ptr(), idx.numel(), self.n_experts, n_sms, out.data_ptr(),
                                        _stream(idx)))
         return out[-1], out

@@ -173,7 +173,11 @@ class Planner:
             return out
         # With a process group the counts have to be summed over the ranks between histogram and
         # LP (lplb/planner.py:214-216); LP and redirect then run as one plan on the summed counts.
-        local_workload, _by_sm = self.count_workload(idx, n_sms)
+        # (the histogram's table is kept per stream like the plan's other buffers)
+        table = ws.get("group_counts")
+        if table is None or table.device != idx.device:
+            table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32, device=idx.device)
+        local_workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
         workload = local_workload.clone()
         if not self.deep_ep_initialized:
             torch.distributed.all_reduce(workload, group=self.ep_group)
