@@ -43,6 +43,11 @@ namespace lplb {
 
 constexpr int kPreferredSlices = 64;   // short batches: slices of 1024, 2048, ... indices while this many cover them
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has static LDS besides
+// An LP workgroup's dynamic LDS starts with the areas its (up to four) LP waves work in, then
+// come the staged counts: per wave the pivot rows (2 * kWave doubles) and the assembly tile.
+constexpr size_t plan_lp_area_bytes(int gm) {
+  return 2 * kWave * sizeof(double) + (size_t)(gm >= LPLB_TILE_MIN ? gm * (gm + 4) + gm : 4) * sizeof(float);
+}
 constexpr int kDefaultMaxPolls = 1 << 22;   // a few seconds of polling before a wait gives up
 // LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP
 // wave is bound by instruction issue, so a fifth LP on the same CU would slow two of them
@@ -142,7 +147,7 @@ static size_t plan_lds_bytes(int n_logical, int n_rep, int n_waves, int k) {
 // waves per SIMD: one 16-wave or two 8-wave workgroups per CU), which is what lets the 257
 // workgroups of a [262144 x 8] batch be resident together.
 template <int GM, int DM, bool EXACT, int K, int WAVES>
-__global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) void plan_in_one_launch(PlanArgs a) {
+__global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) void plan_in_one_launch(PlanArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ int rep_of_edge_all[kLpsPerWorkgroup * kWave];
   __shared__ int flags[2];   // [0] the exchange of counts worked, [1] some share will not come
@@ -187,7 +192,11 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     // the counts) and pick the counts up from LDS; the wave after them waits for the
     // slices, fetches the totals the slices have added up in memory and hands them over.
     __shared__ int counts_ready;
-    float *staged = reinterpret_cast<float *>(smem_raw);
+    // dynamic LDS of an LP workgroup: [LP wave][pivot rows | assembly tile], then the counts
+    constexpr size_t kLpArea = plan_lp_area_bytes(GM);
+    static_assert(kLpArea % 16 == 0, "the LP waves' areas keep 16-byte alignment");
+    unsigned char *my_area = smem_raw + (size_t)min(wave_s, kLpsPerWorkgroup - 1) * kLpArea;
+    float *staged = reinterpret_cast<float *>(smem_raw + kLpsPerWorkgroup * kLpArea);
     if (tid == 0)
       counts_ready = 0;
     __syncthreads();
@@ -226,7 +235,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
     if (wave_s < n_lps) {
       // (own-histogram mode: every LP of the batch reads the one staged copy)
       float *mine = a.local_counts ? staged : staged + (size_t)wave_s * sa.staged_stride;
-      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, first_lp + wave_s, mine, rep_of_edge_all + wave_s * kWave);
+      const int n_ok = solve_lp<GM, DM, EXACT, 1>(sa, first_lp + wave_s, mine, rep_of_edge_all + wave_s * kWave,
+                                                  reinterpret_cast<double *>(my_area),
+                                                  reinterpret_cast<float *>(my_area + 2 * kWave * sizeof(double)));
       if (n_ok < 0) {
         // no counts, no solution: tell the slices not to wait for this LP's shares
         const int n_edges = sa.G * sa.D;
@@ -623,7 +634,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 16) ? 4 : 2) 
 // workgroup size that leaves the LP its registers: 128 VGPRs per lane at 16 waves,
 // 256 at 8.
 constexpr int kPlanShapes[][2] = {{8, 1}, {8, 2}, {8, 4}, {16, 1}, {16, 2}, {32, 1}, {32, 2}};
-constexpr int plan_waves(int gm, int dm) { return (gm * dm <= 16 && gm <= 16) ? 16 : 8; }
+constexpr int plan_waves(int gm, int dm) { return (gm * dm <= 16 && gm <= 8) ? 16 : 8; }
 constexpr int plan_max_chunks(int waves) { return waves == 16 ? 8 : 16; }   // longest slice: 8192 indices
 static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
   for (const auto &shape : kPlanShapes)
@@ -814,20 +825,28 @@ template <int GM, int DM, bool EXACT, int W>
 static int launch_plan_shape(PlanArgs &a, hipStream_t s, bool *done) {
   const int k = chunks_per_wave(a.per, W);
   const size_t lds_slices = plan_lds_bytes(a.sh.n_logical, a.n_rep, W, k);
-  const size_t lds_lp = (size_t)min(a.solve.n_units, kLpsPerWorkgroup) * a.solve.n_experts * sizeof(float);
-  if (lds_slices > (size_t)kPlanLdsLimit)
+  // LP workgroups: their waves' working areas, then the counts (one copy per LP if they fit,
+  // else none and the LPs read global memory; own-histogram mode needs one copy in any case)
+  const size_t lp_areas = kLpsPerWorkgroup * plan_lp_area_bytes(GM);
+  const size_t one_copy = (size_t)a.solve.n_experts * sizeof(float);
+  const size_t all_copies = (size_t)min(a.solve.n_units, kLpsPerWorkgroup) * one_copy;
+  size_t lds = max(lds_slices, lp_areas + (a.local_counts ? one_copy : 0));
+  if (lds > (size_t)kPlanLdsLimit)
     return LPLB_OK;
-  a.solve.staged_stride = lds_lp <= lds_slices ? a.solve.n_experts : 0;
-  if (a.local_counts && (size_t)a.solve.n_experts * sizeof(float) > lds_slices)
-    return LPLB_OK;   // the LP takes its counts from LDS in that mode
+  if (lp_areas + all_copies <= max(lds, (size_t)16 * 1024)) {   // (a few KiB more are worth one global round trip less)
+    lds = max(lds, lp_areas + all_copies);
+    a.solve.staged_stride = a.solve.n_experts;
+  } else {
+    a.solve.staged_stride = 0;
+  }
   switch (k) {
-  case 1: return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds_slices, s, done);
-  case 2: return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds_slices, s, done);
-  case 4: return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds_slices, s, done);
-  case 8: return launch_plan_variant<GM, DM, EXACT, 8, W>(a, lds_slices, s, done);
+  case 1: return launch_plan_variant<GM, DM, EXACT, 1, W>(a, lds, s, done);
+  case 2: return launch_plan_variant<GM, DM, EXACT, 2, W>(a, lds, s, done);
+  case 4: return launch_plan_variant<GM, DM, EXACT, 4, W>(a, lds, s, done);
+  case 8: return launch_plan_variant<GM, DM, EXACT, 8, W>(a, lds, s, done);
   default:
     if constexpr (W == 8)
-      return launch_plan_variant<GM, DM, EXACT, 16, W>(a, lds_slices, s, done);
+      return launch_plan_variant<GM, DM, EXACT, 16, W>(a, lds, s, done);
     return LPLB_OK;
   }
 }
@@ -909,7 +928,7 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
     rc = (G == GM && D == DM) ? launch_plan_shape<GM, DM, true, W>(a, s, done)                \
                               : launch_plan_shape<GM, DM, false, W>(a, s, done);
   LPLB_PLAN_CASE_W(8, 1, 16) LPLB_PLAN_CASE_W(8, 1, 8) LPLB_PLAN_CASE_W(8, 2, 16) LPLB_PLAN_CASE_W(8, 2, 8)
-  LPLB_PLAN_CASE_W(8, 4, 8) LPLB_PLAN_CASE_W(16, 1, 16) LPLB_PLAN_CASE_W(16, 1, 8) LPLB_PLAN_CASE_W(16, 2, 8)
+  LPLB_PLAN_CASE_W(8, 4, 8) LPLB_PLAN_CASE_W(16, 1, 8) LPLB_PLAN_CASE_W(16, 2, 8)
   LPLB_PLAN_CASE_W(32, 1, 8) LPLB_PLAN_CASE_W(32, 2, 8)
 #undef LPLB_PLAN_CASE_W
   return rc;

@@ -15,10 +15,12 @@ template <int GM, int DM, bool EXACT, int ROWS>
 __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   extern __shared__ float staged_all[];   // a.staged_stride floats per LP of this wave
   __shared__ int rep_of_edge[kWave];
+  __shared__ __attribute__((aligned(16))) double pivot_rows[2 * kWave];
+  __shared__ __attribute__((aligned(16))) float tile[assembly_tile_floats<GM>()];
   if (blockIdx.x == 0 && threadIdx.x == 0)
     atomicAdd(a.avail, a.n_units);
   const int first_unit = blockIdx.x * ROWS;
-  const int n_ok = solve_lp<GM, DM, EXACT, ROWS>(a, first_unit, staged_all, rep_of_edge);
+  const int n_ok = solve_lp<GM, DM, EXACT, ROWS>(a, first_unit, staged_all, rep_of_edge, pivot_rows, tile);
   const int n_mine = min(max(a.n_units - first_unit, 0), ROWS);
   if (threadIdx.x == 0 && n_ok < n_mine)
     atomicAdd(a.avail, n_ok - n_mine);
@@ -67,10 +69,14 @@ static int dispatch(const SolveArgs &a, hipStream_t s) {
     launch_solver<GM, DM>(a, s);                                               \
     return LPLB_OK;                                                            \
   }
+#ifdef LPLB_PROBE_G   // (compile-time experiments: one shape only)
+  LPLB_CASE(LPLB_PROBE_G, LPLB_PROBE_D)
+#else
   LPLB_CASE(8, 1) LPLB_CASE(8, 2) LPLB_CASE(8, 4) LPLB_CASE(8, 8)
   LPLB_CASE(16, 1) LPLB_CASE(16, 2) LPLB_CASE(16, 4) LPLB_CASE(16, 8)
   LPLB_CASE(32, 1) LPLB_CASE(32, 2) LPLB_CASE(32, 4)
   LPLB_CASE(64, 1)
+#endif
 #undef LPLB_CASE
   return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
 }

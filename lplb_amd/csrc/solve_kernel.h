@@ -34,6 +34,16 @@
 
 namespace lplb {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+#ifndef LPLB_ROWLDS_MIN
+#define LPLB_ROWLDS_MIN 16
+#endif
+#ifndef LPLB_TILE_MIN
+#define LPLB_TILE_MIN 32
+#endif
+#ifndef LPLB_CHUNK
+#define LPLB_CHUNK 8
+#endif
 
 struct SolveArgs {
   const int32_t *workload;   // [n_inst][n_experts]
@@ -175,6 +185,11 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, uint32_
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// From 32 ranks on a lane's row of S is put together in LDS instead of registers: floats the
+// caller provides per wave (row i at i * (GM + 4), so that 16-byte reads of different lanes'
+// rows fall into different banks; then GM floats for a broadcast copy of v).
+template <int GM> constexpr int assembly_tile_floats() { return GM >= LPLB_TILE_MIN ? GM * (GM + 4) + GM : 4; }
+
 // GM, DM: register-array sizes (group size and replica slots rounded up).
 // EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
 // constant; otherwise rows and columns G..GM-1 of the normal-equation system are
@@ -185,14 +200,17 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, uint32_
 //   first_unit     LP (instance * n_group + group) of the wave's first row
 //   staged_counts  LDS, ROWS * a.staged_stride floats (unused if the stride is 0)
 //   rep_of_edge    LDS, kWave ints
+//   pivot_rows     LDS, 2 * kWave doubles of this wave, 16-byte aligned (one LP per wave only)
+//   tile           LDS, assembly_tile_floats<GM>() floats of this wave, 16-byte aligned (32 ranks or more)
 // Returns how many of the wave's LPs passed the feasibility test (same value in
 // every lane); the caller adds it to a.avail.  -1: the counts the caller promised through
 // a.counts_ready never came; nothing was solved or stored.
 template <int GM, int DM, bool EXACT, int ROWS>
 __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged_counts_of_wave,
-                               int *rep_of_edge) {
+                               int *rep_of_edge, double *pivot_rows, float *tile) {
   constexpr int WL = Layout<ROWS>::kWidth;   // lanes of one LP
   static_assert(ROWS == 1 || (ROWS == 4 && GM <= kRowLanes && GM * DM <= kRowLanes), "an LP must fit its lanes");
+  static_assert(GM % 8 == 0, "pivot rows are read from LDS eight columns at a time");
   constexpr int T = WL / GM;         // lanes that share the work of one rank's b_i
   constexpr int NE = 2 * DM;         // replica edges that touch one rank
   constexpr int KB = ROWS == 1 ? 4 : 16;   // fixed-expert counts a lane prefetches for b_i
@@ -336,14 +354,20 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   }
   // Selectors for assembling my row of S: 1 on my own column, -1 on the column
   // of each edge's other end.
-  float mask[NE][GM], diag_mask[GM];
+  // (From 32 ranks on the selectors alone would be 160 registers: there the row is put
+  // together in LDS instead, see kTileAssembly below.)
+  constexpr bool kTileAssembly = ROWS == 1 && GM >= LPLB_TILE_MIN;
+  constexpr int GS = kTileAssembly ? 1 : GM;
+  float mask[NE][GS], diag_mask[GS];
 #pragma unroll
-  for (int c = 0; c < GM; ++c) {
+  for (int c = 0; c < GS; ++c) {
     diag_mask[c] = (lane == c) ? 1.0f : 0.0f;
 #pragma unroll
     for (int e = 0; e < NE; ++e)
       mask[e][c] = (oth[e] == c) ? -1.0f : 0.0f;
   }
+  float *my_tile_row = tile + (lane < GM ? lane : GM - 1) * (GM + 4);
+  float *v_copy = tile + GM * (GM + 4);
 
   LPLB_STAMP(3);
   // b_i = -(load of the experts that cannot move), minilp.cu:223-234
@@ -417,15 +441,48 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     double S[GM];
     const double dst = (double)st, dkv = (double)kappa * (double)v;
     const float st_col = is_rank ? st : 0.0f;
-    static_for<GM>([&](auto cc) {
-      constexpr int c = decltype(cc)::value;
-      float t = diag_mask[c] * lam_sum;
+    if constexpr (kTileAssembly) {
+      // The Laplacian part of my row: zero it, subtract every edge's weight at the column of
+      // its other end, add the diagonal (LDS float adds, no return value: they queue up in
+      // program order, so each entry is the same sum, in the same order, as with selectors),
+      // read it back.  A lane touches only its own row.  v of every rank comes back from a
+      // copy in LDS, four ranks per read from a wave-uniform address.
+      const f32x4 zero{0.0f, 0.0f, 0.0f, 0.0f};
+      if (lane < GM) {
 #pragma unroll
-      for (int e = 0; e < NE; ++e)
-        t = __builtin_fmaf(mask[e][c], lam_e[e], t);
-      const double base = EXACT ? dst : (double)lp_bcast<ROWS, c>(st_col) * row_on;
-      S[c] = __builtin_fma(dkv, (double)lp_bcast<ROWS, c>(v), base) + (double)t;
-    });
+        for (int c4 = 0; c4 < GM / 4; ++c4)
+          reinterpret_cast<f32x4 *>(my_tile_row)[c4] = zero;
+        v_copy[lane] = v;
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+          __hip_atomic_fetch_add(my_tile_row + oth[e], -lam_e[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        __hip_atomic_fetch_add(my_tile_row + lane, lam_sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      static_for<GM / 4>([&](auto c4c) {
+        constexpr int c4 = decltype(c4c)::value;
+        const f32x4 t4 = reinterpret_cast<const f32x4 *>(my_tile_row)[c4];
+        const f32x4 v4 = reinterpret_cast<const f32x4 *>(v_copy)[c4];
+        const float t[4] = {t4.x, t4.y, t4.z, t4.w}, vc[4] = {v4.x, v4.y, v4.z, v4.w};
+        static_for<4>([&](auto uu) {
+          constexpr int u = decltype(uu)::value, c = 4 * c4 + u;
+          const double base = EXACT ? dst : (double)lp_bcast<ROWS, c>(st_col) * row_on;
+          S[c] = __builtin_fma(dkv, (double)vc[u], base) + (double)t[u];
+        });
+      });
+    } else {
+      static_for<GM>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        float t = diag_mask[c] * lam_sum;
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+          t = __builtin_fmaf(mask[e][c], lam_e[e], t);
+        const double base = EXACT ? dst : (double)lp_bcast<ROWS, c>(st_col) * row_on;
+        S[c] = __builtin_fma(dkv, (double)lp_bcast<ROWS, c>(v), base) + (double)t;
+      });
+    }
     double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
 
     if (step == 0) LPLB_STAMP(6);
@@ -436,32 +493,99 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // The only serial chain is pivot -> reciprocal -> f -> entry (c+1, c+1) -> next
     // pivot; it is written out in that order, with the rest of column step c (which
     // nothing waits for) placed between the links of the next reciprocal, because
-    // the compiler keeps the order it is given here.  (Broadcasting the far columns
-    // of row c through LDS instead of v_readlane halves their instruction count at
-    // 32 ranks, but puts an LDS write -> read round trip into every step of the chain:
-    // measured 45 us against 34 us.  Computing the next pivot one step ahead from three
-    // more broadcasts, in uniform arithmetic, gives bit-identical results and takes the
-    // vector update out of the chain, but costs 9 instructions per pivot and was slower
-    // at 8 ranks, 7.8 us against 7.6 us: at 4.7 clocks per instruction the sweep is
-    // bound by instruction issue more than by the chain.)
+    // the compiler keeps the order it is given here.  (Computing the next pivot one step
+    // ahead from three more broadcasts, in uniform arithmetic, gives bit-identical results
+    // and takes the vector update out of the chain, but costs 9 instructions per pivot and
+    // was slower at 8 ranks.)
     // A lane's own multiple must be zero.  Rather than selecting on the chain (f is the
     // link between reciprocal and update), the lane's diagonal entry is cleared as soon
     // as it has been read as the pivot, one step ahead.
     double my_pivot = 1.0;
     double pivot = lp_bcast<ROWS, 0>(S[0]);
     double rinv = rcp_f64(pivot);
+    // One LP per wave, 16 ranks or more: the entries of pivot row c that the other rows need, S[c][c2] for
+    // c2 > c, are not fetched from lane c one by one (two v_readlane each).  The part of S
+    // that is still being eliminated stays symmetric (up to rounding), so they are also
+    // column c as it is spread over the lanes, S[c2][c] in lane c2: one LDS write of that
+    // register puts the whole row into LDS, and reads from a wave-uniform address hand two
+    // entries at a time to every lane.  LDS instructions do not take the vector ALU's issue
+    // slots, which are what bounds a lone wave.  Column c + 1 is final right after the first
+    // update of step c; it is written then, so the round trip through LDS overlaps the rest
+    // of step c and the reciprocal of the next pivot and is not part of the serial chain.
+    // Two buffers take turns, so a step's reads need not all be issued before the next write.
+    // (Measured: 32 ranks 31.5 -> 12.6 us per LP, 16 ranks 12.6 -> 11.8 us; at 8 ranks the row is
+    // so short that the broadcasts through scalar registers are faster, 7.5 against 7.9 us.)
+    constexpr bool kRowFromLds = ROWS == 1 && GM >= LPLB_ROWLDS_MIN;
+    constexpr int kChunk = LPLB_CHUNK;                       // columns per batch of LDS reads (GM is a multiple)
+    constexpr int kChunks = GM / kChunk;
+    constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
+    // chunk q of the row in buffer `parity`: columns 8 q .. 8 q + 7, four 16-byte reads
+    auto load_chunk = [&](int parity, int q, double (&buf)[kChunk]) {
+      const double2 *src = reinterpret_cast<const double2 *>(pivot_rows + parity * kWave + q * kChunk);
+#pragma unroll
+      for (int j = 0; j < kChunk / 2; ++j) {
+        const double2 both = src[j];
+        buf[2 * j] = both.x;
+        buf[2 * j + 1] = both.y;
+      }
+      // The reads stay where they are written, ahead of their use: left alone, the compiler
+      // moves each one down to the instruction that needs it (fewer live registers) and the
+      // wave then waits out every LDS round trip.
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // The first chunk a step needs is fetched during the step before, right after the column
+    // has been written (two sets of registers take turns).
+    double head[2][kChunk];
+    auto publish_column = [&](auto cc) {
+      constexpr int c = decltype(cc)::value;
+      if constexpr (kRowFromLds && c < GM) {
+        pivot_rows[(c % 2) * kWave + lane] = S[c];   // (every lane writes: no branch; lanes >= GM are never read)
+        __builtin_amdgcn_wave_barrier();
+        if constexpr (c + 1 < GM)
+          load_chunk(c % 2, (c + 1) / kChunk, head[c % 2]);
+      }
+    };
+    publish_column(std::integral_constant<int, 0>{});
     S[0] = (lane == 0) ? 0.0 : S[0];
     static_for<GM>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
+      constexpr int q0 = (c + 1) / kChunk;          // chunk of column c + 1
+      double body[kBodySets][kChunk];
+#ifdef LPLB_STEP_FENCE
+      if constexpr (kRowFromLds)
+        __builtin_amdgcn_sched_barrier(0);
+#endif
+      // S[c2] -= f * (row c)[c2]
       auto clear = [&](auto c2c, double f) {
         constexpr int c2 = decltype(c2c)::value;
-        if constexpr (c2 < GM)
-          S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+#ifdef LPLB_FENCE_ALL
+        if constexpr (kRowFromLds && c2 % LPLB_FENCE_ALL == 0)
+          __builtin_amdgcn_sched_barrier(0);
+#endif
+        if constexpr (c2 < GM) {
+          if constexpr (!kRowFromLds) {
+            S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+          } else if constexpr (c2 / kChunk == q0) {
+            S[c2] = __builtin_fma(-f, head[c % 2][c2 % kChunk], S[c2]);
+          } else {
+            // entering a new chunk: fetch the one after it, and keep the compiler from pulling
+            // every later fetch up here (the rows would not fit the registers)
+            if constexpr (c2 % kChunk == 0 && kBodySets == 2) {
+              __builtin_amdgcn_sched_barrier(0);
+              if constexpr (c2 / kChunk + 1 < kChunks)
+                load_chunk(c % 2, c2 / kChunk + 1, body[(c2 / kChunk + 1) % kBodySets]);
+            }
+            S[c2] = __builtin_fma(-f, body[(c2 / kChunk) % kBodySets][c2 % kChunk], S[c2]);
+          }
+        }
       };
       my_pivot = lp_set_lane<ROWS, c>(my_pivot, pivot, lane);
       const double f = S[c] * rinv;   // multiple of row c to subtract from my row (0 in lane c)
       double next_pivot = 1.0, estimate = 1.0, error = 0.0;
+      if constexpr (kRowFromLds && q0 + 1 < kChunks)
+        load_chunk(c % 2, q0 + 1, body[(q0 + 1) % kBodySets]);
       clear(std::integral_constant<int, c + 1>{}, f);
+      publish_column(std::integral_constant<int, c + 1>{});
       if constexpr (c + 1 < GM) {
         next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
         estimate = __builtin_amdgcn_rcp(next_pivot);
@@ -481,7 +605,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         constexpr int k = decltype(kk)::value;
         // From 32 ranks on a row's broadcasts would fill the scalar registers if the
         // compiler hoisted them all; fence them off in groups of eight columns.
-        if constexpr (GM >= 32 && k % 8 == 0)
+        if constexpr (!kRowFromLds && GM >= 32 && k % 8 == 0)
           __builtin_amdgcn_sched_barrier(0);
         clear(std::integral_constant<int, c + 5 + k>{}, f);
       });
