@@ -36,7 +36,7 @@ namespace lplb {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 #ifndef LPLB_ROWLDS_MIN
-#define LPLB_ROWLDS_MIN 16
+#define LPLB_ROWLDS_MIN 8
 #endif
 #ifndef LPLB_TILE_MIN
 #define LPLB_TILE_MIN 32
@@ -503,7 +503,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     double my_pivot = 1.0;
     double pivot = lp_bcast<ROWS, 0>(S[0]);
     double rinv = rcp_f64(pivot);
-    // One LP per wave, 16 ranks or more: the entries of pivot row c that the other rows need, S[c][c2] for
+    // One LP per wave: the entries of pivot row c that the other rows need, S[c][c2] for
     // c2 > c, are not fetched from lane c one by one (two v_readlane each).  The part of S
     // that is still being eliminated stays symmetric (up to rounding), so they are also
     // column c as it is spread over the lanes, S[c2][c] in lane c2: one LDS write of that
@@ -513,9 +513,10 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // update of step c; it is written then, so the round trip through LDS overlaps the rest
     // of step c and the reciprocal of the next pivot and is not part of the serial chain.
     // Two buffers take turns, so a step's reads need not all be issued before the next write.
-    // (Measured: 32 ranks 31.5 -> 12.6 us per LP, 16 ranks 12.6 -> 11.8 us; at 8 ranks the row is
-    // so short that the broadcasts through scalar registers are faster, 7.5 against 7.9 us.)
-    constexpr bool kRowFromLds = ROWS == 1 && GM >= LPLB_ROWLDS_MIN;
+    // (Measured per LP: 32 ranks 31.5 -> 22.7 us, 16 ranks 12.6 -> 11.4 us, 8 ranks 7.5 -> 7.2 us.  The
+    // padded 8-rank variants keep the scalar broadcasts: inside the one-launch plan they have
+    // no register to spare at four waves per SIMD.)
+    constexpr bool kRowFromLds = ROWS == 1 && (GM >= 16 || (GM >= LPLB_ROWLDS_MIN && EXACT));
     constexpr int kChunk = LPLB_CHUNK;                       // columns per batch of LDS reads (GM is a multiple)
     constexpr int kChunks = GM / kChunk;
     constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
