@@ -46,7 +46,7 @@ constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kerne
 // An LP workgroup's dynamic LDS starts with the areas its (up to four) LP waves work in, then
 // come the staged counts: per wave the pivot rows (2 * kWave doubles) and the assembly tile.
 constexpr size_t plan_lp_area_bytes(int gm) {
-  return 2 * kWave * sizeof(double) + (size_t)(gm >= LPLB_TILE_MIN ? gm * (gm + 4) + gm : 4) * sizeof(float);
+  return 2 * kWave * sizeof(double) + (size_t)(gm >= kTileAssemblyMin ? gm * (gm + 4) + gm : 4) * sizeof(float);
 }
 constexpr int kDefaultMaxPolls = 1 << 22;   // a few seconds of polling before a wait gives up
 // LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP
@@ -212,7 +212,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
         // Poll the batch's totals until every expert's words say that all slices have
         // added theirs.
         bool complete = false;
-        for (int polls = 0; polls < a.max_polls && !complete; ++polls) {
+        for (int polls = 0; polls < a.max_polls && !complete && !poisoned; ++polls) {   // (switched off: no slice will publish)
           bool all_in = true;
           for (int e = lane; e < nl; e += kWave) {
             int32_t tokens, slices;
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
           if (!complete)
             __builtin_amdgcn_s_sleep(2);
         }
-        if (!complete && lane == 0)
+        if (!complete && !poisoned && lane == 0)
           give_up(a);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)

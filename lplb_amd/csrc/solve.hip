@@ -69,14 +69,10 @@ static int dispatch(const SolveArgs &a, hipStream_t s) {
     launch_solver<GM, DM>(a, s);                                               \
     return LPLB_OK;                                                            \
   }
-#ifdef LPLB_PROBE_G   // (compile-time experiments: one shape only)
-  LPLB_CASE(LPLB_PROBE_G, LPLB_PROBE_D)
-#else
   LPLB_CASE(8, 1) LPLB_CASE(8, 2) LPLB_CASE(8, 4) LPLB_CASE(8, 8)
   LPLB_CASE(16, 1) LPLB_CASE(16, 2) LPLB_CASE(16, 4) LPLB_CASE(16, 8)
   LPLB_CASE(32, 1) LPLB_CASE(32, 2) LPLB_CASE(32, 4)
   LPLB_CASE(64, 1)
-#endif
 #undef LPLB_CASE
   return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
 }

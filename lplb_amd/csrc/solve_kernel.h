@@ -35,15 +35,9 @@
 namespace lplb {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-#ifndef LPLB_ROWLDS_MIN
-#define LPLB_ROWLDS_MIN 8
-#endif
-#ifndef LPLB_TILE_MIN
-#define LPLB_TILE_MIN 32
-#endif
-#ifndef LPLB_CHUNK
-#define LPLB_CHUNK 8
-#endif
+// Group sizes from which the elimination takes its pivot rows from LDS (exact-fit variants; padded
+// ones from 16), and from which a lane's row of S is put together in LDS instead of registers.
+constexpr int kRowsFromLdsMin = 8, kTileAssemblyMin = 32;
 
 struct SolveArgs {
   const int32_t *workload;   // [n_inst][n_experts]
@@ -188,7 +182,7 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, uint32_
 // From 32 ranks on a lane's row of S is put together in LDS instead of registers: floats the
 // caller provides per wave (row i at i * (GM + 4), so that 16-byte reads of different lanes'
 // rows fall into different banks; then GM floats for a broadcast copy of v).
-template <int GM> constexpr int assembly_tile_floats() { return GM >= LPLB_TILE_MIN ? GM * (GM + 4) + GM : 4; }
+template <int GM> constexpr int assembly_tile_floats() { return GM >= kTileAssemblyMin ? GM * (GM + 4) + GM : 4; }
 
 // GM, DM: register-array sizes (group size and replica slots rounded up).
 // EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
@@ -356,7 +350,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   // of each edge's other end.
   // (From 32 ranks on the selectors alone would be 160 registers: there the row is put
   // together in LDS instead, see kTileAssembly below.)
-  constexpr bool kTileAssembly = ROWS == 1 && GM >= LPLB_TILE_MIN;
+  constexpr bool kTileAssembly = ROWS == 1 && GM >= kTileAssemblyMin;
   constexpr int GS = kTileAssembly ? 1 : GM;
   float mask[NE][GS], diag_mask[GS];
 #pragma unroll
@@ -516,8 +510,8 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // (Measured per LP: 32 ranks 31.5 -> 22.7 us, 16 ranks 12.6 -> 11.4 us, 8 ranks 7.5 -> 7.2 us.  The
     // padded 8-rank variants keep the scalar broadcasts: inside the one-launch plan they have
     // no register to spare at four waves per SIMD.)
-    constexpr bool kRowFromLds = ROWS == 1 && (GM >= 16 || (GM >= LPLB_ROWLDS_MIN && EXACT));
-    constexpr int kChunk = LPLB_CHUNK;                       // columns per batch of LDS reads (GM is a multiple)
+    constexpr bool kRowFromLds = ROWS == 1 && (GM >= 16 || (GM >= kRowsFromLdsMin && EXACT));
+    constexpr int kChunk = 8;                       // columns per batch of LDS reads (GM is a multiple)
     constexpr int kChunks = GM / kChunk;
     constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
     // chunk q of the row in buffer `parity`: columns 8 q .. 8 q + 7, four 16-byte reads
@@ -547,22 +541,14 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
       }
     };
     publish_column(std::integral_constant<int, 0>{});
-    S[0] = (lane == 0) ? 0.0 : S[0];
+    S[0] = lp_set_lane<ROWS, 0>(S[0], 0.0, lane);
     static_for<GM>([&](auto cc) {
       constexpr int c = decltype(cc)::value;
       constexpr int q0 = (c + 1) / kChunk;          // chunk of column c + 1
       double body[kBodySets][kChunk];
-#ifdef LPLB_STEP_FENCE
-      if constexpr (kRowFromLds)
-        __builtin_amdgcn_sched_barrier(0);
-#endif
       // S[c2] -= f * (row c)[c2]
       auto clear = [&](auto c2c, double f) {
         constexpr int c2 = decltype(c2c)::value;
-#ifdef LPLB_FENCE_ALL
-        if constexpr (kRowFromLds && c2 % LPLB_FENCE_ALL == 0)
-          __builtin_amdgcn_sched_barrier(0);
-#endif
         if constexpr (c2 < GM) {
           if constexpr (!kRowFromLds) {
             S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
@@ -590,7 +576,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
       if constexpr (c + 1 < GM) {
         next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
         estimate = __builtin_amdgcn_rcp(next_pivot);
-        S[c + 1] = (lane == c + 1) ? 0.0 : S[c + 1];
+        S[c + 1] = lp_set_lane<ROWS, c + 1>(S[c + 1], 0.0, lane);
       }
       rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
       clear(std::integral_constant<int, c + 2>{}, f);
