@@ -194,7 +194,7 @@ template <int GM> constexpr int assembly_tile_floats() { return GM >= kTileAssem
 //   first_unit     LP (instance * n_group + group) of the wave's first row
 //   staged_counts  LDS, ROWS * a.staged_stride floats (unused if the stride is 0)
 //   rep_of_edge    LDS, kWave ints
-//   pivot_rows     LDS, 2 * kWave doubles of this wave, 16-byte aligned (one LP per wave only)
+//   pivot_rows     LDS, 2 * kWave doubles of this wave, 16-byte aligned
 //   tile           LDS, assembly_tile_floats<GM>() floats of this wave, 16-byte aligned (32 ranks or more)
 // Returns how many of the wave's LPs passed the feasibility test (same value in
 // every lane); the caller adds it to a.avail.  -1: the counts the caller promised through
@@ -507,16 +507,17 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // update of step c; it is written then, so the round trip through LDS overlaps the rest
     // of step c and the reciprocal of the next pivot and is not part of the serial chain.
     // Two buffers take turns, so a step's reads need not all be issued before the next write.
-    // (Measured per LP: 32 ranks 31.5 -> 22.7 us, 16 ranks 12.6 -> 11.4 us, 8 ranks 7.5 -> 7.2 us.  The
+    // (Measured per LP: 32 ranks 31.5 -> 22.2 us, 16 ranks 12.6 -> 11.2 us, 8 ranks 7.5 -> 7.2 us; four
+    // LPs per wave, each 16-lane row reading its own LP's column: 16384 LPs 30.9 -> 27.6 us.  The
     // padded 8-rank variants keep the scalar broadcasts: inside the one-launch plan they have
     // no register to spare at four waves per SIMD.)
-    constexpr bool kRowFromLds = ROWS == 1 && (GM >= 16 || (GM >= kRowsFromLdsMin && EXACT));
+    constexpr bool kRowFromLds = (ROWS == 1 && (GM >= 16 || (GM >= kRowsFromLdsMin && EXACT))) || ROWS == 4;
     constexpr int kChunk = 8;                       // columns per batch of LDS reads (GM is a multiple)
     constexpr int kChunks = GM / kChunk;
     constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
     // chunk q of the row in buffer `parity`: columns 8 q .. 8 q + 7, four 16-byte reads
     auto load_chunk = [&](int parity, int q, double (&buf)[kChunk]) {
-      const double2 *src = reinterpret_cast<const double2 *>(pivot_rows + parity * kWave + q * kChunk);
+      const double2 *src = reinterpret_cast<const double2 *>(pivot_rows + parity * kWave + lane0 + q * kChunk);
 #pragma unroll
       for (int j = 0; j < kChunk / 2; ++j) {
         const double2 both = src[j];
@@ -534,7 +535,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     auto publish_column = [&](auto cc) {
       constexpr int c = decltype(cc)::value;
       if constexpr (kRowFromLds && c < GM) {
-        pivot_rows[(c % 2) * kWave + lane] = S[c];   // (every lane writes: no branch; lanes >= GM are never read)
+        pivot_rows[(c % 2) * kWave + lane0 + lane] = S[c];   // (every lane writes: no branch; lanes >= GM are never read)
         __builtin_amdgcn_wave_barrier();
         if constexpr (c + 1 < GM)
           load_chunk(c % 2, (c + 1) / kChunk, head[c % 2]);
