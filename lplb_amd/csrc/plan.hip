@@ -41,7 +41,10 @@
 
 namespace lplb {
 
-constexpr int kPreferredSlices = 64;   // short batches: slices of 1024, 2048, ... indices while this many cover them
+#ifndef LPLB_PREFERRED_SLICES
+#define LPLB_PREFERRED_SLICES 64
+#endif
+constexpr int kPreferredSlices = LPLB_PREFERRED_SLICES;   // short batches: slices of 1024, 2048, ... indices while this many cover them
 constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kernel has static LDS besides
 // An LP workgroup's dynamic LDS starts with the areas its (up to four) LP waves work in, then
 // come the staged counts: per wave the pivot rows (2 * kWave doubles) and the assembly tile.
