@@ -173,14 +173,24 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   // The batch's tokens of expert e and the number of slices that have contributed: the copies
   // added up (all loads in flight together); complete once every slice has arrived.
   auto batch_totals = [&](int e, int32_t &tokens, int32_t &slices) {
-    unsigned long long v[kTotalCopies];
-#pragma unroll
-    for (int k = 0; k < kTotalCopies; ++k)
-      v[k] = agent_load(totals_acc + (k & (a.n_copies - 1)) * nl + e);
     unsigned long long sum = 0;
+    if (a.n_copies <= 4) {   // (short batches: a quarter of the loads per look)
+      unsigned long long v[4];
 #pragma unroll
-    for (int k = 0; k < kTotalCopies; ++k)
-      sum += k < a.n_copies ? v[k] : 0ull;
+      for (int k = 0; k < 4; ++k)
+        v[k] = agent_load(totals_acc + (k & (a.n_copies - 1)) * nl + e);
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        sum += k < a.n_copies ? v[k] : 0ull;
+    } else {
+      unsigned long long v[kTotalCopies];
+#pragma unroll
+      for (int k = 0; k < kTotalCopies; ++k)
+        v[k] = agent_load(totals_acc + (k & (a.n_copies - 1)) * nl + e);
+#pragma unroll
+      for (int k = 0; k < kTotalCopies; ++k)
+        sum += k < a.n_copies ? v[k] : 0ull;
+    }
     tokens = (int32_t)(sum >> 32);
     slices = (int32_t)(uint32_t)sum;
   };
