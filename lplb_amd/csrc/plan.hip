@@ -68,7 +68,8 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   kArrivalCopies copies of a striped counter (plan_sync.h);
 //   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits with
 //   tag = (launch tag << 2) | 1 (valid) or 2 (there will be none); a word with another
-//   launch's tag is "not there yet";
+//   launch's tag is "not there yet"; up to kShareCopies copies, kMaxShares words apart: polls of
+//   one line queue up in memory, so slice s polls copy s % copies;
 //   from kTotalsAt: two sets of partial histograms of the batch, [p][copy][n_logical] 8-byte
 //   words with the tokens in the high half and the number of slices that have contributed in
 //   the low half (one atomic add delivers both, so whoever polls the words needs no second
@@ -77,8 +78,8 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   kTotalCopies; more copies cost whoever adds them up more than they save: measured);
 //   whoever needs the batch's tokens per expert adds the copies up.
 constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8;
-constexpr int kSharesAt = 16, kMaxShares = 1024;
-constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares, kMaxTotals = 1024, kTotalCopies = 16;
+constexpr int kSharesAt = 16, kMaxShares = 1024, kShareCopies = 8;
+constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares * kShareCopies, kMaxTotals = 1024, kTotalCopies = 16;
 constexpr int kTotalsWords = kTotalCopies * kMaxTotals;   // 8-byte words of one set
 constexpr int kArrivedAt = kTotalsAt + 2 * 2 * kTotalsWords;   // [2][kArrivalCopies][kArrivalCopyInts]
 constexpr int kSlotInts = kArrivedAt + 2 * kArrivalCopies * kArrivalCopyInts, kSyncSlots = 8;
@@ -96,6 +97,7 @@ struct PlanArgs {
   int n_slices, n_lp_workgroups;
   int n_copies;          // partial histograms of the batch: a power of two, at most kTotalCopies
   int n_arrival_copies;  // copies of the arrival counter: a power of two, at most kArrivalCopies
+  int n_share_copies;    // copies of the LP's shares: a power of two, at most kShareCopies
   int expected_slices;   // = n_slices unless a fault is injected
   int max_polls;
   const int32_t *o2r, *phy2log;
@@ -255,7 +257,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
         // no counts, no solution: tell the slices not to wait for this LP's shares
         const int n_edges = sa.G * sa.D;
         for (int j = lane; j < n_edges; j += kWave)
-          agent_store(shares + (int64_t)(first_lp + wave_s) * n_edges + j, (unsigned long long)tag_none << 32);
+          for (int k = 0; k < a.n_share_copies; ++k)
+            agent_store(shares + (int64_t)k * kMaxShares + (int64_t)(first_lp + wave_s) * n_edges + j,
+                        (unsigned long long)tag_none << 32);
       } else if (lane == 0 && n_ok > 0 && !poisoned) {
         atomicAdd(a.avail, n_ok);
       }
@@ -578,7 +582,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
       unsigned long long word = 0;
       int polls = 0;
       uint32_t tag = 0;
-      while ((tag = (uint32_t)((word = agent_load(shares + s.ep_rank * a.sh.D + s.d)) >> 32)) != tag_valid &&
+      while ((tag = (uint32_t)((word = agent_load(shares + (slice & (a.n_share_copies - 1)) * kMaxShares + s.ep_rank * a.sh.D + s.d)) >> 32)) != tag_valid &&
              tag != tag_none && ++polls < a.max_polls)
         __builtin_amdgcn_s_sleep(2);
       if (tag == tag_valid) {
@@ -814,6 +818,8 @@ static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *don
   PlanSlot &ps = d->slots[slot];
   a.sync = d->sync + (size_t)slot * kSlotInts;
   a.solve.tagged_result = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
+  a.solve.tagged_copies = a.n_share_copies;
+  a.solve.tagged_stride = kMaxShares;
   a.expected_slices = a.n_slices + g_fault_extra_slices.exchange(0);
   const int fault_polls = g_fault_max_polls.exchange(0);
   a.max_polls = fault_polls > 0 ? fault_polls : kDefaultMaxPolls;
@@ -925,6 +931,9 @@ static int try_one_launch(const int64_t *idx, int64_t n_elements, const int32_t 
   a.n_copies = 1;
   while (a.n_copies < kTotalCopies && a.n_copies * 16 < a.n_slices)
     a.n_copies *= 2;
+  a.n_share_copies = 1;
+  while (a.n_share_copies < kShareCopies && a.n_share_copies * 8 < a.n_slices)
+    a.n_share_copies *= 2;
   a.n_arrival_copies = 1;
   while (a.n_arrival_copies < kArrivalCopies && a.n_arrival_copies * 32 < a.n_slices)
     a.n_arrival_copies *= 2;

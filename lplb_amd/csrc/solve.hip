@@ -109,7 +109,7 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
   a.workload = workloads; a.gw_out = global_workloads; a.r2o = r2o; a.phy2log = phy2log;
   a.avail = avail_num; a.result = results; a.n_group = n_group; a.G = group_size;
   a.D = dup_per_rank; a.C = n_experts_per_var; a.n_fixed = n_experts_fixed;
-  a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps; a.tagged_result = nullptr; a.tag_valid = 0; a.counts_ready = nullptr;
+  a.n_experts = (int)n_experts; a.step_rule = step_rule; a.n_steps = n_steps; a.tagged_result = nullptr; a.tag_valid = 0; a.tagged_copies = 0; a.tagged_stride = 0; a.counts_ready = nullptr;
 #ifdef LPLB_PHASE_CLOCKS
   a.clocks = g_phase_clocks;
 #else

@@ -52,6 +52,7 @@ struct SolveArgs {
                              // wave's LP into staged_counts (as floats) and a.workload is not read
   unsigned long long *tagged_result;  // or null: a copy of a.result for other workgroups of the same launch,
   uint32_t tag_valid;                 // each value written through to memory as (tag_valid << 32) | its bits
+  int tagged_copies, tagged_stride;   // ... tagged_copies times, tagged_stride words apart (the pollers spread over the copies)
                                       // (the caller writes tag_valid + 1 for "no result: use the neutral fallback")
   long long *clocks;         // debug builds: wall-clock stamps of wave 0, lane 0 (else null)
 };
@@ -172,11 +173,13 @@ template <int ROWS, int W> __device__ inline float lp_max(float v) {
 
 // Stores a share, and if asked also the copy other workgroups of the running kernel
 // poll: the high word says "valid, from this launch", so value and flag arrive in one 8-byte store.
-__device__ inline void store_share(float *p, unsigned long long *tagged, uint32_t tag, int64_t i, float v) {
+__device__ inline void store_share(float *p, unsigned long long *tagged, uint32_t tag, int copies, int stride,
+                                   int64_t i, float v) {
   p[i] = v;
   if (tagged)
-    __hip_atomic_store(tagged + i, ((unsigned long long)tag << 32) | __builtin_bit_cast(uint32_t, v),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int k = 0; k < copies; ++k)
+      __hip_atomic_store(tagged + (int64_t)k * stride + i, ((unsigned long long)tag << 32) | __builtin_bit_cast(uint32_t, v),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // From 32 ranks on a lane's row of S is put together in LDS instead of registers: floats the
@@ -657,7 +660,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
                   (double)res < 0.05;
   const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
   if (is_edge && unit_on)
-    store_share(a.result, a.tagged_result, a.tag_valid, (int64_t)unit * n + lane, ok ? xo : 0.5f);
+    store_share(a.result, a.tagged_result, a.tag_valid, a.tagged_copies, a.tagged_stride, (int64_t)unit * n + lane, ok ? xo : 0.5f);
   // Normalised counts of this group, for the caller.
   if (a.gw_out && unit_on) {
     float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;
