@@ -95,6 +95,14 @@ class KernelTimer:
         self.used += 1
         self.lib.lplb_time_next_launch(a, b)
 
+    def take(self, n):
+        """The next n pairs as two arrays of events, for the library's *_series calls."""
+        pairs = self.pairs[self.used:self.used + n]
+        assert len(pairs) == n
+        self.used += n
+        arr = self.ct.c_void_p * n
+        return arr(*[a.value for a, _ in pairs]), arr(*[b.value for _, b in pairs])
+
     def times_us(self, torch):
         torch.cuda.synchronize()
         out = []
@@ -237,44 +245,72 @@ def main() -> None:
         total, by = solver.count_idx(b, roof_blocks)
         tables.append(by)
     o_w, _ = solver.solve(tables[0][-1].view(1, G, L), r2o, sweep_p2l, avail)
+    prepared = solver.prepare_mapping(o2r, sweep_p2l)        # once per mapping, as Planner does
+
     def redirect(i, n_blocks=roof_blocks, table=None):
-        rc = lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), (table if table is not None else tables[i]).data_ptr(),
-                              o2r.data_ptr(), sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, n_blocks,
-                              bufs_out[i].data_ptr(), None, stream)
-        assert rc == 0
+        rc = lib.lplb_map_idx_prepared(bufs_in[i].data_ptr(), o_w.data_ptr(),
+                                       (table if table is not None else tables[i]).data_ptr(), prepared.data_ptr(), n_idx,
+                                       1, G, D, C, P, n_blocks, bufs_out[i].data_ptr(), None, stream)
+        assert rc == 0, lib.lplb_last_error()
 
     reps = args.roofline_reps
     for i in range(n_buf):
         redirect(i)
-    # The same bytes through a plain copy kernel are the practical ceiling on this box.  The two
-    # kernels take turns, launch by launch, so that clock ramps and whatever else drifts during
-    # the run treat them alike.
-    timer = KernelTimer(lib, 2 * reps * n_buf)
-    for i in range(n_buf):
         assert lib.lplb_copy_calibration(bufs_in[i].data_ptr(), bufs_out[i].data_ptr(), n_idx, stream) == 0
     torch.cuda.synchronize()
+    # Each launch is timed by its kernel's own begin/end timestamps (what a kernel trace reports).  The launches
+    # come from a loop inside the library: issued one by one from Python, one launch in ten reads about 4 us
+    # longer, redirect and copy alike, which the same launches issued from compiled code do not show.  The same
+    # bytes through a plain copy kernel are the practical ceiling on this box; the two kernels take turns, block
+    # of n_buf launches by block, so that whatever drifts during the run treats them alike.
+    n_series = n_buf
+    timer = KernelTimer(lib, 2 * reps * n_series)
+    ptrs = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    series_in, series_by, series_out = ptrs(bufs_in), ptrs(tables), ptrs(bufs_out)
+    half = n_buf // 2
+    copy_in, copy_out = ptrs(bufs_in[half:] + bufs_in[:half]), ptrs(bufs_out[half:] + bufs_out[:half])
+    red_slots, copy_slots = [], []
     for _ in range(reps):
-        for i in range(n_buf):
-            timer.arm()
-            redirect(i)
-            timer.arm()
-            assert lib.lplb_copy_calibration(bufs_in[(i + n_buf // 2) % n_buf].data_ptr(),
-                                             bufs_out[(i + n_buf // 2) % n_buf].data_ptr(), n_idx, stream) == 0
+        for which, slots in (("redirect", red_slots), ("copy", copy_slots)):
+            starts, stops = timer.take(n_series)
+            if which == "redirect":
+                rc = lib.lplb_map_idx_prepared_series(series_in, o_w.data_ptr(), series_by, prepared.data_ptr(), n_idx, 1, G,
+                                                      D, C, P, roof_blocks, series_out, n_series, starts, stops, stream)
+            else:
+                rc = lib.lplb_copy_calibration_series(copy_in, copy_out, n_idx, n_series, starts, stops, stream)
+            assert rc == 0, lib.lplb_last_error()
+            slots.append(timer.used)
     both_us = timer.times_us(torch)
-    red_us, copy_us = both_us[0::2], both_us[1::2]
+    red_us = np.concatenate([both_us[e - n_series:e] for e in red_slots])
+    copy_us = np.concatenate([both_us[e - n_series:e] for e in copy_slots])
     red_avg = float(red_us.mean())
     alg_bytes = n_idx * REDIRECT_BYTES_PER_INDEX
     achieved = alg_bytes / (red_avg * 1e-6) / 1e9
     copy_gbs = alg_bytes / (float(copy_us.mean()) * 1e-6) / 1e9
+    # the same launches back to back with one event pair around each block: sustained rate, gaps between
+    # kernels included
+    burst = []
+    for _ in range(max(4, reps // 2)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        assert lib.lplb_map_idx_prepared_series(series_in, o_w.data_ptr(), series_by, prepared.data_ptr(), n_idx, 1, G, D, C,
+                                                P, roof_blocks, series_out, n_series, None, None, stream) == 0
+        e1.record()
+        torch.cuda.synchronize()
+        burst.append(e0.elapsed_time(e1) * 1e3 / n_series)
     traffic, traffic_commit = measured_redirect_traffic()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "traffic_measured_at_commit": traffic_commit,
-                "kernel": "redirect_indices",
-                "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64, {roof_blocks} slices",
+                "kernel": "redirect_pairs",
+                "workload": f"sweep_redirect [{sweep.indices.shape[0]} x {sweep.indices.shape[1]}] int64, {roof_blocks} slices, "
+                            "mapping tables prepared once (lplb_map_idx_prepared)",
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
-                "p50_launch_us": round(pct(red_us, 50), 2), "distinct_buffer_pairs": n_buf,
+                "p50_launch_us": round(pct(red_us, 50), 2), "p99_launch_us": round(pct(red_us, 99), 2),
+                "launches_timed": int(red_us.size), "distinct_buffer_pairs": n_buf,
+                "back_to_back_us_per_launch": round(float(np.median(burst)), 2),
                 "copy_kernel_GBs_same_bytes": round(copy_gbs, 1),
+                "copy_kernel_avg_launch_us": round(float(copy_us.mean()), 2),
                 "frac_of_copy_kernel": round(achieved / copy_gbs, 4)}
     extras["redirect_tokens_per_s"] = round(n_idx / (red_avg * 1e-6), 1)
 
@@ -291,6 +327,16 @@ def main() -> None:
                 redirect(i, n_sms, cu_tables[i])
         extras["redirect_sweep_us_one_slice_per_cu"] = round(float(cu_timer.times_us(torch).mean()), 2)
         cu_timer.close()
+        # the reference's own call (o2r and phy2log instead of a prepared table: every workgroup builds the tables)
+        up_timer = KernelTimer(lib, 4 * n_buf)
+        for r in range(4 * n_buf):
+            i = r % n_buf
+            up_timer.arm()
+            assert lib.lplb_map_idx(bufs_in[i].data_ptr(), o_w.data_ptr(), tables[i].data_ptr(), o2r.data_ptr(),
+                                    sweep_p2l.data_ptr(), n_idx, 1, G, D, C, P, roof_blocks, bufs_out[i].data_ptr(), None,
+                                    stream) == 0
+        extras["redirect_sweep_us_without_prepared_table"] = round(float(up_timer.times_us(torch).mean()), 2)
+        up_timer.close()
 
         # histogram at the sweep shape (8 B per index)
         def hist(i):

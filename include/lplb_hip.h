@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 4
+#define LPLB_ABI_VERSION 5
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -55,12 +55,35 @@ void lplb_time_next_launch(void *start_event, void *stop_event);
 
 /*
  * Measurement aid, no counterpart in the reference: a plain streaming copy of
- * n_elements int64 (even count) from src to dst.  Its achieved bandwidth is the
+ * n_elements int64 (even count, 16-byte aligned) from src to dst.  Its achieved bandwidth is the
  * practical ceiling the redirect kernel is compared with, and its known traffic
  * (8 bytes read + 8 written per element) calibrates the profiler's byte counters.
  */
 int lplb_copy_calibration(const int64_t *src, int64_t *dst, int64_t n_elements,
                           lplb_stream_t stream);
+
+/*
+ * Measurement aids, no counterpart in the reference: n_launches calls of
+ * lplb_copy_calibration / lplb_map_idx_prepared issued from one tight loop, launch r on
+ * src[r], dst[r] / idx[r], counts_by_block[r], out[r] (host arrays of n_launches device
+ * pointers; the other arguments as for the single call, physical_counts not written), the
+ * kernel of launch r recording its own begin and end into start_events[r] and
+ * stop_events[r] (hipEvent_t, as for lplb_time_next_launch; either array may be NULL).
+ * For benchmarks written in an interpreted language: per-launch durations taken from a
+ * Python loop showed a tail (one launch in ten 4 us longer) that the same launches issued
+ * from compiled code do not have.
+ */
+int lplb_copy_calibration_series(const int64_t *const *src, int64_t *const *dst,
+                                 int64_t n_elements, int n_launches,
+                                 void *const *start_events, void *const *stop_events,
+                                 lplb_stream_t stream);
+int lplb_map_idx_prepared_series(const int64_t *const *idx, const float *o_weight,
+                                 const int32_t *const *counts_by_block, const void *prepared,
+                                 int64_t n_elements, int n_group, int group_size,
+                                 int dup_per_rank, int n_combined_experts, int n_local_experts,
+                                 int n_blocks, int64_t *const *out, int n_launches,
+                                 void *const *start_events, void *const *stop_events,
+                                 lplb_stream_t stream);
 
 /*
  * Per-expert token histogram with an inclusive prefix over slices.
@@ -158,6 +181,36 @@ int lplb_map_idx(const int64_t *idx, const float *o_weight,
                  int group_size, int dup_per_rank, int n_combined_experts,
                  int n_local_experts, int n_blocks, int64_t *out,
                  int32_t *physical_counts, lplb_stream_t stream);
+
+/*
+ * The part of the redirect's tables that depends on the mapping only, built once per
+ * mapping instead of by every workgroup of every batch.  The reference rebuilds these
+ * tables (where each logical expert's original and replica sit) in every block of every
+ * launch, minilp.cu:466-496; they change only when phy2log does
+ * (lplb/planner.py:115-182, update_redundancy_mapping).
+ *
+ * lplb_prepared_mapping_bytes   size of the table for a shape (-1: bad shape)
+ * lplb_prepare_mapping          fills `prepared` (device memory of the caller's, 16-byte
+ *                               aligned, at least that many bytes) from o2r and phy2log;
+ *                               one small kernel on `stream`.  The table is opaque; it
+ *                               stays valid until phy2log, o2r or the shape change.
+ *                               LPLB_EUNSUPPORTED beyond 511 replicated expert sets or
+ *                               32767 physical experts.
+ * lplb_map_idx_prepared         lplb_map_idx with the table in place of o2r and phy2log:
+ *                               same arguments otherwise, same results bit for bit.
+ */
+int64_t lplb_prepared_mapping_bytes(int n_group, int group_size, int dup_per_rank,
+                                    int n_combined_experts, int n_local_experts);
+int lplb_prepare_mapping(const int32_t *o2r, const int32_t *phy2log, int n_group,
+                         int group_size, int dup_per_rank, int n_combined_experts,
+                         int n_local_experts, void *prepared, int64_t prepared_bytes,
+                         lplb_stream_t stream);
+int lplb_map_idx_prepared(const int64_t *idx, const float *o_weight,
+                          const int32_t *counts_by_block, const void *prepared,
+                          int64_t n_elements, int n_group, int group_size,
+                          int dup_per_rank, int n_combined_experts, int n_local_experts,
+                          int n_blocks, int64_t *out, int32_t *physical_counts,
+                          lplb_stream_t stream);
 
 /*
  * One batch's whole plan in a single call: what Planner.run does with three

@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1
@@ -34,10 +34,15 @@ _SIGNATURES = {
     "lplb_last_error": (ctypes.c_char_p, []),
     "lplb_time_next_launch": (None, [_vp, _vp]),
     "lplb_copy_calibration": (_i, [_vp, _vp, _i64, _vp]),
+    "lplb_copy_calibration_series": (_i, [_vp, _vp, _i64, _i, _vp, _vp, _vp]),
+    "lplb_map_idx_prepared_series": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "lplb_prepared_mapping_bytes": (_i64, [_i, _i, _i, _i, _i]),
+    "lplb_prepare_mapping": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
+    "lplb_map_idx_prepared": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_plan_set_cooperative": (_i, [_i]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
     "lplb_plan_one_launch_count": (_i, [_vp]),
@@ -100,9 +105,14 @@ def plan_one_launch_count() -> int:
     return count.value
 
 
+class UnsupportedShape(RuntimeError):
+    """The library has no kernel for this shape (LPLB_EUNSUPPORTED)."""
+
+
 def _check(rc: int) -> None:
     if rc != 0:
-        raise RuntimeError(f"lplb_hip error {rc}: {load().lplb_last_error().decode()}")
+        kind = UnsupportedShape if rc == 2 else RuntimeError
+        raise kind(f"lplb_hip error {rc}: {load().lplb_last_error().decode()}")
 
 
 def _require(cond: bool, what: str) -> None:
@@ -244,7 +254,9 @@ class CompiledSolver:
     # -- csrc/plugin.cpp:602-660 -------------------------------------------------
     def map_idx(self, mapping_idx: torch.Tensor, o_weight: torch.Tensor, local_workload_split_by_sm: torch.Tensor,
                 o2r: torch.Tensor, phy2log: torch.Tensor, n_sms: int, block_dim: int = 256,
-                physical_counts: torch.Tensor | None = None) -> torch.Tensor:
+                physical_counts: torch.Tensor | None = None, prepared: torch.Tensor | None = None) -> torch.Tensor:
+        """prepared: optional table from prepare_mapping(o2r, phy2log) (no counterpart in the reference,
+        which rebuilds it in every block); the result is the same with and without it."""
         _require(mapping_idx.dtype == torch.int64, "mapping_idx.dtype == int64")
         _require(mapping_idx.is_cuda, "mapping_idx.device().is_cuda()")
         _require(mapping_idx.is_contiguous(), "mapping_idx.is_contiguous()")
@@ -266,6 +278,16 @@ class CompiledSolver:
         _require(block_dim == 256, "slices are aligned to 256 indices")
         self._check_physical_counts(physical_counts)
         out = torch.empty_like(mapping_idx)
+        if prepared is not None:
+            _require(prepared.dtype == torch.int32 and prepared.is_cuda and prepared.is_contiguous()
+                     and prepared.numel() * 4 >= self.prepared_mapping_bytes(), "prepared is a table from prepare_mapping")
+            _check(self.lib.lplb_map_idx_prepared(mapping_idx.data_ptr(), o_weight.data_ptr(), by_sm.data_ptr(),
+                                                  prepared.data_ptr(), mapping_idx.numel(), self.n_group,
+                                                  self.group_size, self.dup_per_rank, self.n_combined_experts,
+                                                  self.n_local_experts, n_sms, out.data_ptr(),
+                                                  physical_counts.data_ptr() if physical_counts is not None else None,
+                                                  _stream(mapping_idx)))
+            return out
         _check(self.lib.lplb_map_idx(mapping_idx.data_ptr(), o_weight.data_ptr(), by_sm.data_ptr(), o2r.data_ptr(),
                                      phy2log.data_ptr(), mapping_idx.numel(), self.n_group, self.group_size,
                                      self.dup_per_rank, self.n_combined_experts, self.n_local_experts, n_sms,
@@ -273,6 +295,27 @@ class CompiledSolver:
                                      physical_counts.data_ptr() if physical_counts is not None else None,
                                      _stream(mapping_idx)))
         return out
+
+    def prepared_mapping_bytes(self) -> int:
+        n = self.lib.lplb_prepared_mapping_bytes(self.n_group, self.group_size, self.dup_per_rank,
+                                                 self.n_combined_experts, self.n_local_experts)
+        _require(n > 0, "a shape the prepared table can describe")
+        return n
+
+    def prepare_mapping(self, o2r: torch.Tensor, phy2log: torch.Tensor) -> torch.Tensor:
+        """The mapping-only part of the redirect's tables as an opaque int32 tensor for map_idx(prepared=...);
+        valid until phy2log or o2r change."""
+        _require(o2r.dtype == torch.int32 and o2r.is_cuda and o2r.is_contiguous()
+                 and tuple(o2r.shape) == (self.group_size, self.dup_per_rank), "o2r is a contiguous int32 [G, D] GPU tensor")
+        _require(phy2log.dtype == torch.int32 and phy2log.is_cuda and phy2log.is_contiguous() and phy2log.dim() == 1
+                 and phy2log.size(0) == self.group_size * self.n_group * self.n_local_experts,
+                 "phy2log is a contiguous int32 [n_group * group_size * n_local_experts] GPU tensor")
+        n_bytes = self.prepared_mapping_bytes()
+        table = torch.empty((n_bytes + 3) // 4, dtype=torch.int32, device=phy2log.device)
+        _check(self.lib.lplb_prepare_mapping(o2r.data_ptr(), phy2log.data_ptr(), self.n_group, self.group_size,
+                                             self.dup_per_rank, self.n_combined_experts, self.n_local_experts,
+                                             table.data_ptr(), n_bytes, _stream(phy2log)))
+        return table
 
     def _check_physical_counts(self, t: torch.Tensor | None) -> None:
         """Optional output of map_idx / plan: tokens per physical expert (the bincount of the result)."""

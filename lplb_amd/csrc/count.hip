@@ -26,6 +26,7 @@ __global__ __launch_bounds__(1024) void slice_histogram(
     const int64_t *__restrict__ idx, int64_t n, int n_experts, int64_t per,
     int32_t *__restrict__ counts) {
   extern __shared__ int32_t hist[];
+  fetch_arguments_now(idx, n, n_experts, per, counts);
   const int tid = threadIdx.x, nt = blockDim.x;
   const int p = blockIdx.x;
   for (int e = tid; e < n_experts; e += nt)
@@ -77,6 +78,7 @@ __global__ __launch_bounds__(kScanBands *kScanCols) void prefix_over_slices(
     int32_t *__restrict__ counts, int n_blocks, int n_experts) {
   __shared__ int32_t part[kScanBands][kScanCols];
   __shared__ int32_t carry[kScanCols];
+  fetch_arguments_now(counts, n_blocks, n_experts);
   const int col = threadIdx.x % kScanCols, band = threadIdx.x / kScanCols;
   const int e = blockIdx.x * kScanCols + col;
   const bool live = e < n_experts;

@@ -5,80 +5,32 @@
 
 namespace lplb {
 
-// Per-expert constants of the redirect, one 16-byte LDS read per token.
-struct __attribute__((aligned(16))) ExpertEntry {
-  int32_t total;     // tokens of this expert in the whole index array
-  uint32_t magic;    // floor((2^32 - 1) / total), 0 for total <= 0
-  int32_t expected;  // tokens that stay on the original, trunc(o_weight * total)
-  int32_t original;  // physical slot of the original
-};
-
-// State of one expert inside one wave, one 16-byte LDS read / write per token.
-struct __attribute__((aligned(16))) WaveSlot {
-  int32_t next;             // ordinal of the wave's next token of this expert
-  int32_t unused;
-  unsigned long long bits;  // lanes of the current chunk that hold this expert
-};
-
 // h mod total with C's truncating sign rule.  magic = floor((2^32 - 1) / total) is at
 // least 2^32 / total - 1, so for a <= 2^31: a / total >= a * magic / 2^32 >=
 // a / total - 1/2.  q = mulhi(a, magic) is therefore the true quotient or one less,
 // and one conditional subtract finishes (a 32-bit division per expert instead of one
 // per token).
 // WRAP: the hash 499 k + 41 may have wrapped to negative.
-template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, const ExpertEntry &x) {
+template <bool WRAP> __device__ inline int32_t hashed_mod(int32_t h, int32_t total, uint32_t magic) {
   const uint32_t a = WRAP ? (uint32_t)max(h, -h) : (uint32_t)h;
-  uint32_t r = a - __umulhi(a, x.magic) * (uint32_t)x.total;
-  r = min(r, r - (uint32_t)x.total);           // one conditional subtract
+  uint32_t r = a - __umulhi(a, magic) * (uint32_t)total;
+  r = min(r, r - (uint32_t)total);           // one conditional subtract
   int32_t m = (WRAP && h < 0) ? -(int32_t)r : (int32_t)r;
-  return x.total > 0 ? m : 0;
+  return total > 0 ? m : 0;
 }
 
 constexpr int kMaxWaves = 16;
 typedef int i32x4 __attribute__((ext_vector_type(4)));
-
 
 // The shapes the table build needs.
 struct RedirectShape {
   int n_logical, n_ranks, G, D, C, L, P;
 };
 
-// table / replica / first ordinal of expert e: total tokens t, of which `start` lie
-// before this workgroup's slice.  minilp.cu:466-496.
-__device__ inline void init_entry(ExpertEntry *table, int32_t *replica, int32_t *carry, int e, int32_t t,
-                                  int32_t start) {
-  ExpertEntry x;
-  x.total = t;
-  x.magic = t >= 1 ? 0xffffffffu / (uint32_t)t : 0u;
-  x.expected = t;
-  x.original = -1;
-  table[e] = x;
-  replica[e] = -1;
-  carry[e] = start;
-}
-// Physical slot e holds logical expert le as its original.
-__device__ inline void set_original(ExpertEntry *table, const RedirectShape &sh, int e, int le) {
-  if (le >= 0 && le < sh.n_logical)
-    table[le].original = (e / sh.L) * sh.P + (e % sh.L);
-}
-// Replica slot `local` of EP rank ep_rank copies logical expert le; the copy lives on
-// group rank `host`.
-__device__ inline void set_replica_slot(int32_t *replica, const RedirectShape &sh, int ep_rank, int local, int le,
-                                        int host) {
-  if (le >= 0 && le < sh.n_logical)
-    replica[le] = ((ep_rank / sh.G) * sh.G + host + 1) * sh.P - sh.C * sh.D + local;
-}
-// Tokens of an expert with `total` tokens that stay on its original when the original
+// Tokens of an expert with `total` tokens that stay on the original when the original
 // keeps `share` of them: the fp32 product truncated toward zero (saturating, NaN -> 0).
 __device__ inline int32_t expected_on_original(float share, int32_t total) {
   return __float2int_rz(share * (float)total);
-}
-// Both at once.
-__device__ inline void set_replica(ExpertEntry *table, int32_t *replica, const RedirectShape &sh, int ep_rank,
-                                   int local, int le, float share, int host) {
-  if (le >= 0 && le < sh.n_logical)
-    table[le].expected = expected_on_original(share, table[le].total);
-  set_replica_slot(replica, sh, ep_rank, local, le, host);
 }
 
 // How many of an expert's `total` tokens stay on the original:
@@ -94,67 +46,6 @@ __device__ inline int32_t kept_on_original(int32_t total, int32_t expected) {
     return want;
   const int32_t m = total / 499;
   return 499 * (want > 41 ? min(m, (want - 41 + 498) / 499) : 0);
-}
-
-// Tokens per physical expert, = bincount of the redirect's output, from the tables
-// of any one workgroup: every slot is the original or the replica of its logical expert.
-__device__ inline void emit_physical_counts(const ExpertEntry *table, const int32_t *replica,
-                                            const RedirectShape &sh, const int32_t *phy2log, int32_t *counts,
-                                            int tid, int nt) {
-  for (int i = tid; i < sh.n_ranks * sh.P; i += nt) {
-    const int le = phy2log[i];
-    int32_t v = 0;
-    if (le >= 0 && le < sh.n_logical) {
-      const ExpertEntry x = table[le];
-      const int32_t kept = kept_on_original(x.total, x.expected);
-      if (x.original == i)
-        v = kept;
-      else if (replica[le] == i)
-        v = x.total - kept;
-    }
-    counts[i] = v;
-  }
-}
-
-// One token of a 64-index chunk: lanes holding the same expert find each other
-// through the wave's 64-bit bitmap for that expert; the rank among those peers is a
-// popcount of lower lanes and the last peer advances the wave's ordinal.  Returns
-// the token's hash (499 k + 41) mod total (minilp.cu:505) and, in x, its expert's
-// entry; neither is defined for e < 0.  All lanes of the wave call it together and
-// put a wave barrier between chunks.  It does not read x.expected, so it may run
-// before the LP's shares are known.
-template <bool WRAP>
-__device__ inline int32_t hash_of_token(int e, WaveSlot *mine, const ExpertEntry *table, unsigned long long my_bit,
-                                        ExpertEntry &x) {
-  const bool valid = e >= 0;
-  if (valid)
-    atomicOr(&mine[e].bits, my_bit);
-  int32_t h = 0;
-  if (valid) {
-    const i32x4 sraw = *reinterpret_cast<const i32x4 *>(&mine[e]);
-    const i32x4 xraw = *reinterpret_cast<const i32x4 *>(&table[e]);
-    const uint32_t peers_lo = (uint32_t)sraw.z, peers_hi = (uint32_t)sraw.w;
-    const int rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
-    const int cnt = __popc(peers_lo) + __popc(peers_hi);
-    const int32_t k = sraw.x + rank;
-    x.total = xraw.x; x.magic = (uint32_t)xraw.y; x.expected = xraw.z; x.original = xraw.w;
-    h = hashed_mod<WRAP>((int32_t)((uint32_t)k * 499u + 41u), x);
-    if (rank == cnt - 1)   // last peer: advance the ordinal, clear the bitmap
-      *reinterpret_cast<i32x4 *>(&mine[e]) = i32x4{k + 1, 0, 0, 0};
-  }
-  return h;
-}
-
-// The physical expert of a token of expert e with hash h (-1 for e < 0).
-template <bool WRAP>
-__device__ inline int64_t redirect_token(int e, WaveSlot *mine, const ExpertEntry *table, const int32_t *replica,
-                                         unsigned long long my_bit) {
-  ExpertEntry x;
-  const int32_t h = hash_of_token<WRAP>(e, mine, table, my_bit, x);
-  int64_t o = -1;
-  if (e >= 0)
-    o = h >= x.expected ? replica[e] : x.original;
-  return o;
 }
 
 // ---------------------------------------------------------------------------
@@ -196,10 +87,7 @@ constexpr int rank_record_bytes(int k) { return 2 * k * (int)sizeof(ChunkSlot) +
 // !WRAP: k < 2^24 and 499 k + 41 < 2^31 (the caller guarantees it).
 template <bool WRAP> __device__ inline int32_t ordinal_hash(int32_t k, int32_t total, uint32_t magic) {
   if constexpr (WRAP) {
-    ExpertEntry x;
-    x.total = total;
-    x.magic = magic;
-    return hashed_mod<true>((int32_t)((uint32_t)k * 499u + 41u), x);
+    return hashed_mod<true>((int32_t)((uint32_t)k * 499u + 41u), total, magic);
   } else {
     const uint32_t a = __umul24((uint32_t)k, 499u) + 41u;
     const uint32_t r = a - __umulhi(a, magic) * (uint32_t)total;   // true remainder, or that plus total

@@ -12,7 +12,7 @@ import functools
 import numpy as np
 import torch
 
-from ._native import CompiledSolver, _stream
+from ._native import CompiledSolver, UnsupportedShape, _stream
 from .mapping import build_redundancy_mapping
 
 
@@ -83,6 +83,7 @@ class Planner:
         self.deep_ep_initialized = False
         self._solver: CompiledSolver | None = None
         self._run_buffers: dict = {}
+        self._prepared: tuple | None = None   # (key of the mapping it was built from, table or None)
 
     @property
     def solver(self) -> CompiledSolver:
@@ -137,13 +138,26 @@ class Planner:
             torch.distributed.all_reduce(workload, group=self.ep_group)
         return self.solver.solve(workload, self.r2o, self.phy2log, avail_counter)
 
+    def _prepared_mapping(self) -> torch.Tensor | None:
+        """The redirect's mapping-only tables (which the reference rebuilds in every block of every launch,
+        minilp.cu:466-496), built once per phy2log; None for shapes the prepared form does not cover."""
+        key = (self.phy2log.data_ptr(), self.phy2log._version, self.o2r.data_ptr(), self.o2r._version)
+        if self._prepared is None or self._prepared[0] != key:
+            try:
+                table = self.solver.prepare_mapping(self.o2r, self.phy2log)
+            except UnsupportedShape:
+                table = None
+            self._prepared = (key, table)
+        return self._prepared[1]
+
     def weighted_select_target(self, idx: torch.Tensor, o_weight: torch.Tensor,
                                local_workload_by_sm: torch.Tensor, n_sms: int) -> torch.Tensor:
         """Map logical expert ids to physical ones according to ``o_weight``.
 
         :return: int64, same shape as ``idx``, values in [-1, n_routed_experts).
         """
-        return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256)
+        return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256,
+                                   prepared=self._prepared_mapping())
 
     def run(self, idx: torch.Tensor, avail_counter: torch.Tensor, n_sms: int | None = None, *,
             physical_counts: torch.Tensor | None = None) -> torch.Tensor:

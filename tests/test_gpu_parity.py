@@ -78,6 +78,13 @@ def test_map_idx_matches_oracle(cuda, case, n, n_sms):
     np.testing.assert_array_equal(got, want)
     # tokens per physical expert, as the reference's test counts them (tests/test_idx_processing.py:100-101)
     np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
+    # the same through a table prepared once for the mapping
+    table = solver.prepare_mapping(dev(shape.o2r, cuda), dev(phy2log, cuda))
+    phys2 = torch.full((shape.n_physical,), -7, dtype=torch.int32, device=cuda)
+    out2 = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms,
+                          physical_counts=phys2, prepared=table)
+    np.testing.assert_array_equal(out2.cpu().numpy(), want)
+    np.testing.assert_array_equal(phys2.cpu().numpy(), phys.cpu().numpy())
     # reference test's properties (tests/test_idx_processing.py:88-98)
     assert got.min() >= -1 and got.max() < shape.n_physical
     assert np.array_equal(got == -1, idx == -1)
@@ -118,6 +125,10 @@ def test_map_idx_extreme_weights(cuda):
     want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
     np.testing.assert_array_equal(got, want)
     np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
+    table = solver.prepare_mapping(dev(shape.o2r, cuda), dev(phy2log, cuda))
+    got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 64,
+                         prepared=table).cpu().numpy()
+    np.testing.assert_array_equal(got, want)
 
 
 @pytest.mark.parametrize("multiple", [1, 2, 7])
@@ -140,8 +151,9 @@ def test_physical_counts_when_499_divides_a_total(cuda, multiple):
         if trial == 0:
             o_weight[:] = 41.0 / (499 * multiple)      # expected = 41 (or 40): the first hash value is 41
         phys = torch.empty(shape.n_physical, dtype=torch.int32, device=cuda)
+        table = solver.prepare_mapping(dev(shape.o2r, cuda), dev(phy2log, cuda)) if trial % 2 else None
         got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), 32,
-                             physical_counts=phys).cpu().numpy()
+                             physical_counts=phys, prepared=table).cpu().numpy()
         want = oracle.map_idx(idx, o_weight, by_sm.cpu().numpy(), shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
         np.testing.assert_array_equal(got, want)
         np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical))
@@ -179,8 +191,9 @@ def test_count_and_redirect_random_shapes(cuda):
         want_by = oracle.count_idx(idx, n_logical, n_sms)
         np.testing.assert_array_equal(by_sm.cpu().numpy(), want_by, err_msg=f"trial {trial}")
         phys = torch.full((shape.n_physical,), -3, dtype=torch.int32, device=cuda)
+        table = solver.prepare_mapping(dev(shape.o2r, cuda), dev(phy2log, cuda)) if trial % 2 else None
         got = solver.map_idx(d_idx, dev(o_weight, cuda), by_sm, dev(shape.o2r, cuda), dev(phy2log, cuda), n_sms,
-                             physical_counts=phys).cpu().numpy()
+                             physical_counts=phys, prepared=table).cpu().numpy()
         want = oracle.map_idx(idx, o_weight, want_by, shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
         np.testing.assert_array_equal(got, want, err_msg=f"trial {trial}")
         np.testing.assert_array_equal(phys.cpu().numpy(), np.bincount(want[want >= 0], minlength=shape.n_physical),
@@ -1168,6 +1181,49 @@ def test_one_launch_plans_beyond_what_fits_the_gpu_run_as_the_chain(cuda):
     print(f"{as_one_launch} of 60 concurrent plans ran as one launch")
     assert 5 <= as_one_launch <= 60
     assert _native.plan_sync_timeouts() == timeouts_before
+
+
+@pytest.mark.parametrize("n", [2, 4096, 2048 * 2 * 512, 2048 * 2 * 512 + 6, 5_000_002])
+def test_copy_calibration_copies(cuda, n):
+    """The yardstick kernel really moves the bytes it is credited with (whole tiles, ragged ends, more tiles
+    than resident workgroups)."""
+    from lplb_amd import _native
+    lib = _native.load()
+    src = torch.arange(n, dtype=torch.int64, device=cuda) * 7 - 3
+    dst = torch.zeros(n + 2, dtype=torch.int64, device=cuda)
+    assert lib.lplb_copy_calibration(src.data_ptr(), dst.data_ptr(), n, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n], src) and int(dst[n]) == 0 and int(dst[n + 1]) == 0
+
+
+def test_series_aids_equal_single_calls(cuda):
+    """lplb_map_idx_prepared_series / lplb_copy_calibration_series are the single calls in a loop."""
+    import ctypes
+    from lplb_amd import _native
+    lib = _native.load()
+    shape, _, phy2log, _, _ = reference_style_case(*REFERENCE_SOLVE_CASES[0][1:6], seed=3)
+    rng = np.random.default_rng(17)
+    solver = solver_for(shape)
+    o_weight = dev(_random_weights(shape, rng), cuda)
+    d_o2r, d_p2l = dev(shape.o2r, cuda), dev(phy2log, cuda)
+    table = solver.prepare_mapping(d_o2r, d_p2l)
+    n, n_sms = 40960, 20
+    idx = [dev(rng.integers(-1, shape.n_logical, size=n, dtype=np.int64), cuda) for _ in range(3)]
+    by = [solver.count_idx(t, n_sms)[1] for t in idx]
+    want = [solver.map_idx(t, o_weight, b, d_o2r, d_p2l, n_sms) for t, b in zip(idx, by)]
+    out = [torch.full_like(t, -9) for t in idx]
+    ptrs = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+    rc = lib.lplb_map_idx_prepared_series(ptrs(idx), o_weight.data_ptr(), ptrs(by), table.data_ptr(), n, shape.n_group,
+                                          shape.G, shape.D, shape.C, shape.P, n_sms, ptrs(out), 3, None, None, None)
+    assert rc == 0, lib.lplb_last_error()
+    torch.cuda.synchronize()
+    for o, w in zip(out, want):
+        assert torch.equal(o, w)
+    back = [torch.zeros_like(t) for t in idx]
+    assert lib.lplb_copy_calibration_series(ptrs(idx), ptrs(back), n, 3, None, None, None) == 0
+    torch.cuda.synchronize()
+    for o, w in zip(back, idx):
+        assert torch.equal(o, w)
 
 
 def test_kernel_timestamp_hook(cuda):

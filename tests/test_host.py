@@ -190,7 +190,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert sorted(_native.exported_symbols()) == declared
-    assert lib.lplb_abi_version() == _native.ABI_VERSION == 4
+    assert lib.lplb_abi_version() == _native.ABI_VERSION == 5
     header = (ROOT / "include" / "lplb_hip.h").read_text()
     assert f"#define LPLB_ABI_VERSION {_native.ABI_VERSION}" in header
 
