@@ -31,6 +31,7 @@ extern "C" {
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
 #define LPLB_EUNSUPPORTED 2 /* shape outside what the kernels are built for */
 #define LPLB_EHIP 3        /* a HIP runtime call failed */
+#define LPLB_EBUSY 4       /* a resource inside the library is in use by work on another stream */
 
 /* Step-length rules of the affine-scaling iteration. */
 #define LPLB_STEP_REFERENCE_WINDOW 0 /* max over the last 32 columns, as minilp.cu:355-359 does */
@@ -247,15 +248,17 @@ int lplb_map_idx_prepared(const int64_t *idx, const float *o_weight,
  * several (see lplb_plan_set_cooperative).  Every wait inside the kernel is bounded; if one
  * runs out, the launch still completes, with a valid but unbalanced result: the tokens of
  * the slices whose wait ran out go to their experts' original slots (so every entry of
- * `out` still names a slot that holds the token's expert).  The failure is counted
- * (lplb_plan_sync_timeouts) and the caller has to look at that counter before it trusts
- * what else the calls since its last look returned: physical_counts is filled with -1 when
- * the workgroup that writes it is among those that gave up (always the case when the
- * counts of the batch never became complete), the last row of counts_by_block may not have
- * been written, avail_num counts the LPs that were solved, whether or not the slices got to
- * use them.  After such a failure the stream's later plans that would run as one launch
- * send every token to the original slot and count one more failure each, until
- * lplb_plan_sync_timeouts has been called.
+ * `out` still names a slot that holds the token's expert).  avail_num does not vouch for
+ * such a batch: the reference's callers read "avail_num grew by n_group" as "this batch was
+ * balanced" (tests/test_solve.py:58), so the first workgroup that gives up takes the
+ * launch's feasible LPs back out of avail_num and LPs that finish later do not add
+ * themselves; the same holds for every later plan on a block of counters that is switched
+ * off.  The failure is also counted (lplb_plan_poll_timeouts reports the count without
+ * waiting, lplb_plan_sync_timeouts reports it and switches the one-launch form on again).
+ * What else such a call returns: physical_counts is filled with -1 when the workgroup that
+ * writes it is among those that gave up (always the case when the counts of the batch never
+ * became complete) and may otherwise not match `out`; the last row of counts_by_block may
+ * not have been written.
  */
 int lplb_plan(const int64_t *idx, int64_t n_elements,
               const int32_t *global_counts, const int32_t *r2o,
@@ -282,9 +285,17 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
  *
  * Limit: n_blocks * n_logical <= 262144 counters (LPLB_EUNSUPPORTED beyond; e.g. 256
  * slices of 1024 logical experts, 1024 slices of 256).  Every call on a GPU uses that
- * GPU's one table, whatever the stream: calls whose kernels overlap in time on one GPU
- * race on it.  Calls on one stream are ordered and safe.  The table keeps the previous
- * call's contents; nothing in it needs clearing, every row is written before it is read.
+ * GPU's one table, whatever the stream.  Calls on one stream are ordered and safe; a call
+ * on another stream is refused with LPLB_EBUSY while the previous caller's kernels may
+ * still be running (the library records an event of its own behind every call and asks
+ * the runtime about it; it never waits), and for good once a call has been captured into
+ * a graph, whose replays the library cannot see.  Calls replayed from graphs captured on
+ * different streams are the caller's to keep apart.  The table keeps the previous call's
+ * contents; nothing in it needs clearing, every row is written before it is read.
+ * The first call on a device looks the table's address up, creates that event and reads
+ * the kernels' attributes: it has to happen outside a stream capture.  From inside a
+ * capture the runtime cannot be asked about another stream's work, so a call that is being
+ * captured is accepted only on the stream that used the table last.
  */
 int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
                       const int32_t *global_counts, const int32_t *r2o,
@@ -314,6 +325,16 @@ int lplb_plan_set_cooperative(int enabled);
  * to be called while a stream is being captured or while other threads enqueue plans.
  */
 int lplb_plan_sync_timeouts(int *count);
+
+/*
+ * No counterpart in the reference.  The same health report without waiting: a one-thread
+ * kernel on `stream` writes dst[0] = waits that ran out on the current device since the
+ * library was loaded and dst[1] = blocks of counters that are switched off right now.
+ * dst: two int32 in device memory or in pinned host memory (which the caller reads once
+ * work enqueued after this call has completed, or simply at its next look).  Nothing is
+ * cleared or switched on again; that takes lplb_plan_sync_timeouts.
+ */
+int lplb_plan_poll_timeouts(int32_t *dst, lplb_stream_t stream);
 
 /*
  * No counterpart in the reference.  *count receives how many lplb_plan /

@@ -45,6 +45,7 @@ _SIGNATURES = {
     "lplb_map_idx_prepared": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_plan_set_cooperative": (_i, [_i]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
+    "lplb_plan_poll_timeouts": (_i, [_vp, _vp]),
     "lplb_plan_one_launch_count": (_i, [_vp]),
     "lplb_plan_inject_fault": (_i, [_i, _i]),
     "lplb_plan": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
@@ -96,6 +97,14 @@ def plan_sync_timeouts() -> int:
     count = ctypes.c_int(-1)
     _check(load().lplb_plan_sync_timeouts(ctypes.byref(count)))
     return count.value
+
+
+def plan_poll_timeouts(dst: torch.Tensor, stream: int | None = None) -> None:
+    """Enqueue the health report: dst (two int32, on the GPU or in pinned host memory) receives the number of
+    waits that ran out on the current device and the number of blocks of counters switched off."""
+    _require(dst.dtype == torch.int32 and dst.numel() >= 2 and dst.is_contiguous() and (dst.is_cuda or dst.is_pinned()),
+             "dst: two int32 on the GPU or in pinned host memory")
+    _check(load().lplb_plan_poll_timeouts(dst.data_ptr(), stream))
 
 
 def plan_one_launch_count() -> int:

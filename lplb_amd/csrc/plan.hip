@@ -64,6 +64,11 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   [kPoisonAt] non-zero: a wait ran out in this block (see above); [kTimeoutsAt] waits that
 //   ran out since the library was loaded (never cleared);
 //   [kDirtyAt + p] how many words of set p's totals the last launch that used it may have left non-zero;
+//   [kAvailAt + 2 p] (8 bytes) who has touched the caller's counter of feasible LPs in the launch that uses
+//   set p: bit k = LP k was feasible and has been (or is being) added, bit 32 = a wait ran out, so the
+//   batch is not balanced as a whole and whoever set the bit took the LPs added so far back out; an LP
+//   that finds bit 32 set does not add itself.  The reference's callers read "counter == number of
+//   groups" as "this batch was balanced" (tests/test_solve.py:58, scripts/run_ep16_cube8p2e.py:61).
 //   from kArrivedAt: workgroups that have published (slices) or started (LP): per set p,
 //   kArrivalCopies copies of a striped counter (plan_sync.h);
 //   from kSharesAt: the LP's shares as 8-byte words (tag << 32) | float bits with
@@ -77,7 +82,8 @@ constexpr int kLpsPerWorkgroup = 4, kMaxLpWorkgroups = 8;
 //   updates of one address queue up behind each other, so one copy per 16 slices (at most
 //   kTotalCopies; more copies cost whoever adds them up more than they save: measured);
 //   whoever needs the batch's tokens per expert adds the copies up.
-constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8;
+constexpr int kGenAt = 0, kPoisonAt = 1, kTimeoutsAt = 4, kDirtyAt = 8, kAvailAt = 10;
+constexpr unsigned long long kGaveUp = 1ull << 32;
 constexpr int kSharesAt = 16, kMaxShares = 1024, kShareCopies = 8;
 constexpr int kTotalsAt = kSharesAt + 2 * kMaxShares * kShareCopies, kMaxTotals = 1024, kTotalCopies = 16;
 constexpr int kTotalsWords = kTotalCopies * kMaxTotals;   // 8-byte words of one set
@@ -115,10 +121,15 @@ struct PlanArgs {
   int *sync;
 };
 
-// A wait ran out: count it and switch the block of counters off.
-__device__ inline void give_up(const PlanArgs &a) {
+// A wait ran out: count it, switch the block of counters off, and make sure the caller's counter of
+// feasible LPs does not vouch for this batch (the first to give up takes back what the LPs have added).
+__device__ inline void give_up(const PlanArgs &a, unsigned long long *avail_state) {
   agent_add(a.sync + kTimeoutsAt, 1);
   agent_store(a.sync + kPoisonAt, 1);
+  const unsigned long long before = __hip_atomic_fetch_or(avail_state, kGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const int added = __popcll(before & 0xffffffffull);
+  if (!(before & kGaveUp) && added > 0)
+    atomicAdd(a.avail, -added);
 }
 
 // LDS of a slice workgroup: route and histogram per logical expert, a ranking record per
@@ -170,6 +181,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   const uint32_t tag_valid = (((uint32_t)gen + 1u) << 2) | 1u, tag_none = tag_valid + 1u;
   int *arrived_stripes = a.sync + kArrivedAt + parity * (kArrivalCopies * kArrivalCopyInts);
   unsigned long long *shares = reinterpret_cast<unsigned long long *>(a.sync + kSharesAt);
+  unsigned long long *avail_state = reinterpret_cast<unsigned long long *>(a.sync + kAvailAt) + parity;
   unsigned long long *totals_acc =
       reinterpret_cast<unsigned long long *>(a.sync + kTotalsAt) + (size_t)parity * kTotalsWords;   // [n_copies][nl]
   // The batch's tokens of expert e and the number of slices that have contributed: the copies
@@ -223,6 +235,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
     sa.tag_valid = tag_valid;
     if (a.local_counts) {
       sa.counts_ready = &counts_ready;
+      // strictly longer than the poller's own wait (whose polls are each many loads long): the poller is
+      // the one that gives up and says so
+      sa.counts_wait_polls = a.max_polls < (INT32_MAX >> 6) ? a.max_polls << 6 : INT32_MAX;
       if (wave_s == n_lps) {
         // Poll the batch's totals until every expert's words say that all slices have
         // added theirs.
@@ -240,7 +255,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
             __builtin_amdgcn_s_sleep(2);
         }
         if (!complete && !poisoned && lane == 0)
-          give_up(a);
+          give_up(a, avail_state);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (lane == 0)
           __hip_atomic_store(&counts_ready, complete ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -254,14 +269,22 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
                                                   reinterpret_cast<double *>(my_area),
                                                   reinterpret_cast<float *>(my_area + 2 * kWave * sizeof(double)));
       if (n_ok < 0) {
-        // no counts, no solution: tell the slices not to wait for this LP's shares
+        // no counts, no solution: tell the slices not to wait for this LP's shares.  (If it was this wave's
+        // own wait that ran out and not the poller's, nobody has counted the failure yet.)
+        if (lane == 0 && !poisoned &&
+            __hip_atomic_load(&counts_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 2)
+          give_up(a, avail_state);
         const int n_edges = sa.G * sa.D;
         for (int j = lane; j < n_edges; j += kWave)
           for (int k = 0; k < a.n_share_copies; ++k)
             agent_store(shares + (int64_t)k * kMaxShares + (int64_t)(first_lp + wave_s) * n_edges + j,
                         (unsigned long long)tag_none << 32);
       } else if (lane == 0 && n_ok > 0 && !poisoned) {
-        atomicAdd(a.avail, n_ok);
+        // feasible: count it for the caller unless some workgroup has already given up on this batch
+        const unsigned long long before = __hip_atomic_fetch_or(avail_state, 1ull << (first_lp + wave_s), __ATOMIC_RELAXED,
+                                                                 __HIP_MEMORY_SCOPE_AGENT);
+        if (!(before & kGaveUp))
+          atomicAdd(a.avail, n_ok);
       }
     }
     LPLB_PLAN_STAMP(2);
@@ -388,8 +411,10 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
       if (tid < kArrivalCopies * kArrivalStripes)
         agent_store(a.sync + kArrivedAt + ((1 - parity) * kArrivalCopies + tid / kArrivalStripes) * kArrivalCopyInts +
                         (tid % kArrivalStripes) * kArrivalStripeInts, 0);
-      if (tid == 0)
+      if (tid == 0) {
         agent_store(a.sync + kDirtyAt + parity, a.n_copies * nl);
+        agent_store(reinterpret_cast<unsigned long long *>(a.sync + kAvailAt) + (1 - parity), 0ull);
+      }
     }
   }
   __syncthreads();
@@ -482,7 +507,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
                                              a.expected_slices + a.n_lp_workgroups, a.max_polls);
       if (lane == 0) {
         if (!arrived)
-          give_up(a);
+          give_up(a, avail_state);
         else if (slice == 0)
           agent_store(a.sync + kGenAt, (gen + 1) & 0x3fffffff);   // every workgroup has read it by now
         flags[0] = arrived;
@@ -589,7 +614,7 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
         reps[R - 1 - i].expected = expected_on_original(__builtin_bit_cast(float, (uint32_t)word), total[R - 1 - i]);
       } else {
         if (tag != tag_none)
-          give_up(a);
+          give_up(a, avail_state);
         flags[1] = 1;
       }
     }
@@ -672,9 +697,11 @@ static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
 // does not see it.
 struct PlanSlot {
   hipStream_t stream = nullptr;
+  hipEvent_t done = nullptr;    // recorded behind the slot's latest one-launch plan (the library's own: the
+                                // stream handle may be stale by the time somebody asks)
   float cost = 0.0f;            // share of the GPU's resident workgroups its launches take
   bool used = false, captured = false;
-  bool maybe_executing = false; // a launch was enqueued and the stream has not been seen idle since
+  bool maybe_executing = false; // a launch was enqueued and its event has not been seen complete since
 };
 struct PlanDevice {
   int *sync = nullptr;
@@ -706,19 +733,18 @@ static int plan_device(PlanDevice **out) {
   return LPLB_OK;
 }
 
-// May a launch of this slot still be executing?  Asks the runtime whether the slot's stream
-// has work pending (any work: a stream busy with other kernels counts as executing, which
-// only errs towards the chain); never waits.
-// may_ask = false (the calling stream is being captured, and a stream query would break the
-// capture): what is not known to be idle counts as executing.
+// May a launch of this slot still be executing?  Asks the runtime about the event recorded behind the
+// slot's latest plan; never waits and never touches the stream itself (other threads may be capturing
+// on it, or may have destroyed it).  may_ask = false (the calling stream is being captured: no queries
+// from inside a capture): what is not known to be over counts as executing.
 static bool slot_is_executing(PlanDevice &d, int i, bool may_ask) {
   PlanSlot &s = d.slots[i];
   if (!s.used)
     return false;
   if (s.captured)
     return true;
-  if (s.maybe_executing && may_ask && hipStreamQuery(s.stream) != hipErrorNotReady)
-    s.maybe_executing = false;   // idle (or the stream is gone)
+  if (s.maybe_executing && may_ask && s.done != nullptr && hipEventQuery(s.done) != hipErrorNotReady)
+    s.maybe_executing = false;
   return s.maybe_executing;
 }
 
@@ -823,8 +849,14 @@ static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *don
   a.expected_slices = a.n_slices + g_fault_extra_slices.exchange(0);
   const int fault_polls = g_fault_max_polls.exchange(0);
   a.max_polls = fault_polls > 0 ? fault_polls : kDefaultMaxPolls;
+  // The event that says when this launch is over: the slot's own, made at its first launch outside a capture
+  // (a captured launch keeps its share of the GPU for good and needs none).
+  if (!capturing && ps.done == nullptr && hipEventCreateWithFlags(&ps.done, hipEventDisableTiming) != hipSuccess)
+    return fail(LPLB_EHIP, "plan: cannot create an event");
   launch(kernel, dim3(n_workgroups), dim3(WAVES * kWave), lds, s, a);
-  const hipError_t err = hipGetLastError();
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess && !capturing)
+    err = hipEventRecord(ps.done, s);
   if (err != hipSuccess)
     return fail(LPLB_EHIP, "plan: launch failed: %s", hipGetErrorString(err));
   ps.maybe_executing = !capturing;
@@ -990,6 +1022,33 @@ extern "C" int lplb_plan_sync_timeouts(int *count) {
   return LPLB_OK;
 }
 
+namespace lplb {
+// dst[0] = waits that ran out on this device so far, dst[1] = blocks of counters switched off right now
+__global__ void report_plan_health(const int *sync, int32_t *dst) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    int timeouts = 0, off = 0;
+    for (int slot = 0; slot < kSyncSlots; ++slot) {
+      timeouts += agent_load(sync + (size_t)slot * kSlotInts + kTimeoutsAt);
+      off += agent_load(sync + (size_t)slot * kSlotInts + kPoisonAt) != 0;
+    }
+    dst[0] = timeouts;
+    dst[1] = off;
+  }
+}
+} // namespace lplb
+
+extern "C" int lplb_plan_poll_timeouts(int32_t *dst, lplb_stream_t stream) {
+  using namespace lplb;
+  LPLB_REQUIRE(dst != nullptr, LPLB_EINVAL, "plan_poll_timeouts: null pointer");
+  PlanDevice *d = nullptr;
+  const int rc = plan_device(&d);
+  if (rc != LPLB_OK)
+    return rc;
+  launch(report_plan_health, dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream), d->sync, dst);
+  LPLB_HIP_TRY(hipGetLastError());
+  return LPLB_OK;
+}
+
 extern "C" int lplb_plan_one_launch_count(long long *count) {
   LPLB_REQUIRE(count != nullptr, LPLB_EINVAL, "plan_one_launch_count: null pointer");
   *count = lplb::g_one_launch_plans.load(std::memory_order_relaxed);
@@ -1069,21 +1128,33 @@ static int plan_checked(const int64_t *idx, int64_t n_elements, const int32_t *g
 constexpr int64_t kScratchInts = 1 << 18;   // 1 MiB: e.g. 256 slices x 1024 logical experts
 static __device__ __align__(256) int32_t scratch[kScratchInts];
 
-// Device address of `scratch` on the current device, looked up once per device (the
-// array's name is only a host-side handle; threads that race for the first look-up
-// store the same value).
-static int scratch_of_current_device(int32_t **ptr) {
-  static std::atomic<int32_t *> scratch_of[64];
+// Per device: the table's address (the array's name is only a host-side handle: looked up once, at the
+// first call on the device) and who used the table last.  One table serves every stream, so a call from
+// another stream is refused while the last user's kernels may still be running; `done` is recorded
+// behind each call and is made, like the address, at that first call, which therefore has to happen
+// outside a stream capture.  A call captured into a graph keeps the table for its stream for good.
+struct ScratchUse {
+  int32_t *table = nullptr;
+  hipEvent_t done = nullptr;
+  hipStream_t stream = nullptr;
+  bool used = false, captured = false;
+};
+static ScratchUse g_scratch_use[64];
+static std::mutex g_scratch_guard;
+
+static int scratch_of_current_device(ScratchUse **use) {
   int dev = -1;
   LPLB_HIP_TRY(hipGetDevice(&dev));
   LPLB_REQUIRE(dev >= 0 && dev < 64, LPLB_EUNSUPPORTED, "plan_noalloc: device ordinal %d", dev);
-  int32_t *p = scratch_of[dev].load(std::memory_order_acquire);
-  if (!p) {
+  ScratchUse &u = g_scratch_use[dev];
+  if (!u.table) {
+    int32_t *p = nullptr;
     LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
     LPLB_REQUIRE(p != nullptr, LPLB_EHIP, "plan_noalloc: no device address for the slice table");
-    scratch_of[dev].store(p, std::memory_order_release);
+    LPLB_HIP_TRY(hipEventCreateWithFlags(&u.done, hipEventDisableTiming));
+    u.table = p;
   }
-  *ptr = p;
+  *use = &u;
   return LPLB_OK;
 }
 
@@ -1128,19 +1199,41 @@ extern "C" int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
                "plan_noalloc: n_blocks=%d x %lld logical experts = %lld counters exceed the built-in slice table of "
                "%lld; use fewer slices or lplb_plan with a workspace of your own",
                n_blocks, (long long)n_logical, (long long)((int64_t)n_blocks * n_logical), (long long)kScratchInts);
-  int32_t *table = nullptr;
-  int rc = scratch_of_current_device(&table);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capture) != hipSuccess)
+    capture = hipStreamCaptureStatusNone;
+  const bool capturing = capture == hipStreamCaptureStatusActive;
+  std::lock_guard<std::mutex> lock(g_scratch_guard);   // held over the call: check, enqueue and record agree
+  ScratchUse *use = nullptr;
+  int rc = scratch_of_current_device(&use);
   if (rc != LPLB_OK)
     return rc;
+  if (use->used && use->stream != s) {
+    // (from inside a capture the runtime is not asked: what is not known to be over counts as running)
+    const bool busy = use->captured || capturing || hipEventQuery(use->done) == hipErrorNotReady;
+    LPLB_REQUIRE(!busy, LPLB_EBUSY,
+                 "plan_noalloc: the built-in slice table is in use by a plan on another stream%s; wait for it, keep "
+                 "such plans on one stream, or use lplb_plan with a workspace of your own",
+                 use->captured ? " (captured into a graph, which keeps it)" : "");
+  }
+  int32_t *table = use->table;
   // Nothing in the table has to start at zero: every row is written (by the slice that
   // owns it) before anything reads it, and rows beyond n_blocks are never read.
   rc = plan_checked(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
                     n_combined_experts, n_local_experts, n_blocks, table, global_workload, o_weight, avail_num, out,
                     physical_counts, step_rule, n_steps, stream);
-  if (rc != LPLB_OK || local_counts == nullptr)
-    return rc;
-  launch(copy_ints, dim3((unsigned)((n_logical + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
-         table + (int64_t)(n_blocks - 1) * n_logical, local_counts, (int)n_logical);
-  LPLB_HIP_TRY(hipGetLastError());
-  return LPLB_OK;
+  if (rc == LPLB_OK && local_counts != nullptr) {
+    launch(copy_ints, dim3((unsigned)((n_logical + 255) / 256)), dim3(256), 0, s,
+           table + (int64_t)(n_blocks - 1) * n_logical, local_counts, (int)n_logical);
+    if (hipGetLastError() != hipSuccess)
+      rc = fail(LPLB_EHIP, "plan_noalloc: launch failed");
+  }
+  // whatever was enqueued may touch the table, also when a later step of the chain failed
+  use->used = true;
+  use->stream = s;
+  use->captured = use->captured || capturing;
+  if (!capturing && hipEventRecord(use->done, s) != hipSuccess && rc == LPLB_OK)
+    rc = fail(LPLB_EHIP, "plan_noalloc: cannot record an event");
+  return rc;
 }

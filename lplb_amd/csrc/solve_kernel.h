@@ -50,6 +50,7 @@ struct SolveArgs {
   int staged_stride;   // floats of LDS per LP for its counts, 0 = read them from global memory
   const int *counts_ready;   // or null.  LDS flag: once it is non-zero the caller has put the counts of this
                              // wave's LP into staged_counts (as floats) and a.workload is not read
+  int counts_wait_polls;     // how many times to look at that flag before giving up on it
   unsigned long long *tagged_result;  // or null: a copy of a.result for other workgroups of the same launch,
   uint32_t tag_valid;                 // each value written through to memory as (tag_valid << 32) | its bits
   int tagged_copies, tagged_stride;   // ... tagged_copies times, tagged_stride words apart (the pollers spread over the copies)
@@ -271,9 +272,9 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   float out_cnt[KG];
   if (prestaged) {
     // 1 = the counts are staged, 2 = the caller gave up on them; the wait itself is bounded
-    // as well (2^26 polls, seconds), so that this wave ends whatever happens to the flag.
+    // as well, so that this wave ends whatever happens to the flag.
     int ready = 0;
-    for (int polls = 0; polls < (1 << 26); ++polls) {
+    for (int polls = 0; polls < a.counts_wait_polls; ++polls) {
       ready = __hip_atomic_load(a.counts_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (ready != 0)
         break;

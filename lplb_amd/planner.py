@@ -8,10 +8,12 @@ any host synchronisation.
 from __future__ import annotations
 
 import functools
+import warnings
 
 import numpy as np
 import torch
 
+from . import _native
 from ._native import CompiledSolver, UnsupportedShape, _stream
 from .mapping import build_redundancy_mapping
 
@@ -84,6 +86,11 @@ class Planner:
         self._solver: CompiledSolver | None = None
         self._run_buffers: dict = {}
         self._prepared: tuple | None = None   # (key of the mapping it was built from, table or None)
+        # health of the one-launch plan (see _look_at_plan_health)
+        self.health_check_every = 64
+        self.plan_timeouts = 0                # waits between workgroups that ran out on this device, as last seen
+        self._health: torch.Tensor | None = None
+        self._calls_since_health = 0
 
     @property
     def solver(self) -> CompiledSolver:
@@ -159,6 +166,33 @@ class Planner:
         return self.solver.map_idx(idx, o_weight, local_workload_by_sm, self.o2r, self.phy2log, n_sms, 256,
                                    prepared=self._prepared_mapping())
 
+    def _look_at_plan_health(self, idx: torch.Tensor) -> None:
+        """Every ``health_check_every`` calls: read what the report enqueued that many calls ago wrote into pinned
+        host memory (no synchronisation: it has long been written) and enqueue the next report."""
+        self._calls_since_health += 1
+        if self._calls_since_health < self.health_check_every:
+            return
+        self._calls_since_health = 0
+        if self._health is None:
+            self._health = torch.zeros(2, dtype=torch.int32).pin_memory()
+        else:
+            self._handle_plan_health(int(self._health[0]), int(self._health[1]))
+        _native.plan_poll_timeouts(self._health, _stream(idx))
+
+    def _handle_plan_health(self, timeouts: int, switched_off: int) -> None:
+        """A wait between the workgroups of a one-launch plan ran out (a multi-second stall of the GPU, or kernels
+        of the caller's that keep the plan's workgroups from being resident together): such plans leave their
+        tokens on the original slots and do not raise ``avail_counter``; plans on that stream stay that way until
+        the block of counters is switched on again, which is done here (it waits for the device once)."""
+        if timeouts > self.plan_timeouts or switched_off:
+            warnings.warn(f"lplb_amd: {timeouts - self.plan_timeouts} wait(s) between the workgroups of a one-launch plan ran "
+                          f"out since the last look ({switched_off} block(s) of counters switched off); the batches "
+                          "concerned were not balanced (avail_counter was not raised for them); switching the "
+                          "one-launch form on again", RuntimeWarning, stacklevel=3)
+            self.plan_timeouts = timeouts
+            if switched_off:
+                self.plan_timeouts = _native.plan_sync_timeouts()
+
     def run(self, idx: torch.Tensor, avail_counter: torch.Tensor, n_sms: int | None = None, *,
             physical_counts: torch.Tensor | None = None) -> torch.Tensor:
         """Assign a physical expert to every selected logical expert.
@@ -174,12 +208,21 @@ class Planner:
         # run() hands out only the redirected indices, so the plan's other buffers (slice table,
         # shares, normalised counts) are kept per stream and slice count instead of being
         # allocated for every batch; work on one stream is ordered, so reuse is safe there
+        capturing = torch.cuda.is_current_stream_capturing()
         key = (_stream(idx), n_sms)
         ws = self._run_buffers.get(key)
         if ws is None:
             if len(self._run_buffers) >= 16:
-                self._run_buffers.clear()
+                # drop the oldest set of buffers that no captured graph can still be pointing at
+                for old_key, old_ws in self._run_buffers.items():
+                    if not old_ws.get("captured"):
+                        del self._run_buffers[old_key]
+                        break
             ws = self._run_buffers[key] = {}
+        if capturing:
+            ws["captured"] = True
+        else:
+            self._look_at_plan_health(idx)
         if self.ep_group is None:
             # count_workload -> solve_probs -> weighted_select_target in one library call
             out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,

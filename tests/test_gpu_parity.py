@@ -1121,10 +1121,21 @@ def test_one_launch_plan_gives_up_in_a_defined_way(cuda, use_global):
         assert _native.plan_one_launch_count() == launches_before + 1 + later
         np.testing.assert_array_equal(out.cpu().numpy(), stay)
         assert torch.all(phys == -1)
-    # (with the counts supplied the LP needs nothing from the slices and is solved all the same in the
-    # first of the two launches; a launch that finds the block switched off adds nothing)
-    assert int(avail[0]) == (2 if use_global else 1)
+    # The counter of feasible LPs must not vouch for a batch that was not balanced (the reference's callers
+    # assert on it, tests/test_solve.py:58): with the counts supplied the LP is solved all the same in the first
+    # of the two launches, and whichever comes first, its add or the first give-up, the add does not stay; a
+    # launch that finds the block switched off adds nothing.
+    assert int(avail[0]) == 1
+    # the report that does not wait says the same as the synchronous one is about to
+    report = torch.full((2,), -1, dtype=torch.int32, device=cuda)
+    _native.plan_poll_timeouts(report)
+    torch.cuda.synchronize()
+    assert int(report[1]) == 1 and int(report[0]) - timeouts_before >= 64 + 1
     gave_up = _native.plan_sync_timeouts() - timeouts_before      # ... which also switches the block on again
+    pinned = torch.full((2,), -1, dtype=torch.int32).pin_memory()
+    _native.plan_poll_timeouts(pinned)
+    torch.cuda.synchronize()
+    assert int(pinned[1]) == 0 and int(pinned[0]) - timeouts_before == gave_up
     assert gave_up >= 64 + 1, gave_up           # every slice workgroup's wait (and the LP's, if it waited too), and the second plan
     # the next plans on the same stream are healthy
     avail.zero_()
@@ -1136,6 +1147,33 @@ def test_one_launch_plan_gives_up_in_a_defined_way(cuda, use_global):
     assert int(avail[0]) == 3
     assert _native.plan_sync_timeouts() - timeouts_before == gave_up
     assert _native.plan_one_launch_count() == launches_before + 5
+
+
+def test_planner_run_notices_a_wait_that_ran_out(cuda):
+    """Planner.run looks at the health report every few calls without waiting for the GPU; after a forced
+    give-up it warns, switches the one-launch form on again and plans correctly from then on."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    planner = Planner(torch.from_numpy(inp.cfg.r2o), inp.cfg.n_physical, inp.cfg.n_logical, inp.cfg.ep_size, device=cuda)
+    planner.phy2log = t["phy2log"]
+    planner.health_check_every = 2
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    want = planner.run(t["idx"], avail, 256).clone()
+    torch.cuda.synchronize()
+    before = _native.plan_sync_timeouts()
+    planner.plan_timeouts = before
+    print("injecting a wait that cannot be met", flush=True)
+    assert _native.load().lplb_plan_inject_fault(1, 2000) == 0
+    avail.zero_()
+    with pytest.warns(RuntimeWarning, match="not balanced"):
+        for _ in range(8):
+            out = planner.run(t["idx"], avail, 256)
+            torch.cuda.synchronize()
+    assert planner.plan_timeouts > before
+    unbalanced = 8 - int(avail[0])
+    assert 1 <= unbalanced <= 5, unbalanced      # from the give-up to the look that re-armed: two looks at most, two calls apart
+    assert torch.equal(out, want)
+    assert _native.plan_sync_timeouts() == planner.plan_timeouts
 
 
 def test_one_launch_slots_pass_from_stream_to_stream(cuda):

@@ -136,6 +136,39 @@ def test_planner_needs_a_gpu_for_the_kernels():
         p.init_from_deep_ep(None)
 
 
+def test_planner_surfaces_waits_that_ran_out(monkeypatch):
+    """Planner.run looks at the one-launch plan's health report every few calls; a non-zero count must reach the
+    user (a warning, the attribute) and switch the one-launch form on again.  The report itself needs a GPU;
+    what is done with it does not."""
+    from lplb_amd import _native as native
+    p = Planner(torch.from_numpy(topology.RING_8P), 64 + 8, 64, 8, device="cpu")
+    rearmed = []
+    monkeypatch.setattr(native, "plan_sync_timeouts", lambda: rearmed.append(1) or 5)
+    import warnings as w
+    with w.catch_warnings():
+        w.simplefilter("error")
+        p._handle_plan_health(0, 0)                    # healthy: silent
+    assert p.plan_timeouts == 0 and not rearmed
+    with pytest.warns(RuntimeWarning, match="not balanced"):
+        p._handle_plan_health(3, 1)
+    assert rearmed == [1] and p.plan_timeouts == 5     # the synchronous call's own count after re-arming
+    with pytest.warns(RuntimeWarning):
+        p._handle_plan_health(7, 0)                    # counted since, but no block is off: nothing to re-arm
+    assert rearmed == [1] and p.plan_timeouts == 7
+    with w.catch_warnings():
+        w.simplefilter("error")
+        p._handle_plan_health(7, 0)                    # nothing new
+    # the look itself is spaced out and never happens on a CPU planner before the kernels are needed
+    calls = []
+    monkeypatch.setattr(native, "plan_poll_timeouts", lambda dst, stream=None: calls.append(dst))
+    monkeypatch.setattr(torch.Tensor, "pin_memory", lambda self: self)
+    monkeypatch.setattr("lplb_amd.planner._stream", lambda t: 0)
+    p.health_check_every = 4
+    for _ in range(9):
+        p._look_at_plan_health(torch.zeros(1))
+    assert len(calls) == 2 and calls[0] is calls[1] and calls[0].dtype == torch.int32
+
+
 def test_compiled_solver_argument_checks():
     """Same refusals as the reference's extension (csrc/plugin.cpp:494-530, 582-584, 605-628)."""
     s = _native.CompiledSolver(1, 8, 2, 34, 1)

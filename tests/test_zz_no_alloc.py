@@ -120,3 +120,55 @@ def test_plan_noalloc_refuses_what_its_table_cannot_hold(cuda):
     torch.cuda.synchronize()
     want = oracle.count_idx(inp.indices.reshape(-1), shape.n_logical, 1)[-1]
     np.testing.assert_array_equal(o.local.cpu().numpy(), want)
+
+
+def test_plan_noalloc_allocates_nothing_and_replays_from_a_graph(cuda):
+    """What the entry point is for: after a first call (which looks up addresses and attributes), a call
+    leaves torch's allocator as it found it, and a call captured into a HIP graph replays with the same
+    result as the eager call, several times, with other work in between."""
+    lib = _native.load()
+    inp = synth.make_inputs("v3_ep8_cube", mask_fraction=0.05)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    idx = _dev(inp.indices.reshape(-1), cuda)
+    r2o, o2r, p2l = _dev(shape.r2o, cuda), _dev(shape.o2r, cuda), _dev(inp.phy2log, cuda)
+    counts = _dev(inp.global_counts, cuda)
+    eager, replayed = _Outputs(idx.numel(), shape, cuda), _Outputs(idx.numel(), shape, cuda)
+
+    def call(o, stream):
+        rc = lib.lplb_plan_noalloc(_ptr(idx), idx.numel(), _ptr(counts), _ptr(r2o), _ptr(o2r), _ptr(p2l), shape.n_group,
+                                   shape.G, shape.D, shape.C, shape.P, 256, _ptr(o.local), _ptr(o.gw), _ptr(o.o_weight),
+                                   _ptr(o.avail), _ptr(o.out), _ptr(o.physical), 0, 5, VP(stream))
+        assert rc == 0, lib.lplb_last_error()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(eager, side.cuda_stream)                       # warm-up on the stream that will be captured
+        torch.cuda.synchronize()
+        allocated, reserved = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        free_before = torch.cuda.mem_get_info()[0]
+        eager.avail.zero_()
+        call(eager, side.cuda_stream)
+        torch.cuda.synchronize()
+        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (allocated, reserved)
+        assert torch.cuda.mem_get_info()[0] == free_before  # nothing taken from the device behind torch's back either
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):              # (the stream that used the table last: see the header)
+        call(replayed, side.cuda_stream)
+    for replay in range(3):
+        replayed.out.fill_(-7)
+        replayed.physical.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed.out, eager.out) and torch.equal(replayed.physical, eager.physical)
+        assert torch.equal(replayed.o_weight, eager.o_weight) and torch.equal(replayed.local, eager.local)
+        _ = (idx + replay).sum().item()                      # eager work and a synchronisation between replays
+    assert int(replayed.avail[0]) == 3
+    # the captured call keeps the table: another stream is told so instead of racing on it
+    other = torch.cuda.Stream()
+    rc = lib.lplb_plan_noalloc(_ptr(idx), idx.numel(), _ptr(counts), _ptr(r2o), _ptr(o2r), _ptr(p2l), shape.n_group,
+                               shape.G, shape.D, shape.C, shape.P, 256, None, _ptr(eager.gw), _ptr(eager.o_weight),
+                               _ptr(eager.avail), _ptr(eager.out), None, 0, 5, VP(other.cuda_stream))
+    assert rc == 4 and b"another stream" in lib.lplb_last_error()
