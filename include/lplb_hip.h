@@ -287,15 +287,13 @@ int lplb_plan(const int64_t *idx, int64_t n_elements,
  * slices of 1024 logical experts, 1024 slices of 256).  Every call on a GPU uses that
  * GPU's one table, whatever the stream.  Calls on one stream are ordered and safe; a call
  * on another stream is refused with LPLB_EBUSY while the previous caller's kernels may
- * still be running (the library records an event of its own behind every call and asks
- * the runtime about it; it never waits), and for good once a call has been captured into
- * a graph, whose replays the library cannot see.  Calls replayed from graphs captured on
- * different streams are the caller's to keep apart.  The table keeps the previous call's
- * contents; nothing in it needs clearing, every row is written before it is read.
- * The first call on a device looks the table's address up, creates that event and reads
- * the kernels' attributes: it has to happen outside a stream capture.  From inside a
- * capture the runtime cannot be asked about another stream's work, so a call that is being
- * captured is accepted only on the stream that used the table last.
+ * still be running (the last kernel of every call reports its end in a word of pinned host
+ * memory, which the next call looks at; nothing waits), and for good once a call has been
+ * captured into a graph, whose replays the library cannot see.  Calls replayed from graphs
+ * captured on different streams are the caller's to keep apart.  The table keeps the
+ * previous call's contents; nothing in it needs clearing, every row is written before it
+ * is read.  The first call on a device looks the table's address up, sets that word up and
+ * reads the kernels' attributes: it has to happen outside a stream capture.
  */
 int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
                       const int32_t *global_counts, const int32_t *r2o,

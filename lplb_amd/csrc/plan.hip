@@ -119,6 +119,8 @@ struct PlanArgs {
   SolveArgs solve;   // result = the shares (o_weight); workload is replaced by the totals if local_counts
   int local_counts;
   int *sync;
+  int *arrived_word;   // pinned host memory, or null: receives arrived_seq once every workgroup of the launch has arrived
+  int arrived_seq;
 };
 
 // A wait ran out: count it, switch the block of counters off, and make sure the caller's counter of
@@ -167,6 +169,10 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ int rep_of_edge_all[kLpsPerWorkgroup * kWave];
   __shared__ int flags[2];   // [0] the exchange of counts worked, [1] some share will not come
+  fetch_arguments_now(a.idx, a.n, a.per, a.n_slices, a.n_lp_workgroups, a.n_copies, a.n_arrival_copies, a.n_share_copies,
+                      a.expected_slices, a.max_polls, a.o2r, a.phy2log, a.rows, a.row_shift, a.totals, a.out,
+                      a.physical_counts, a.avail, a.sh.n_logical, a.sh.n_ranks, a.sh.G, a.sh.D, a.sh.C, a.sh.L, a.sh.P,
+                      a.n_rep, a.magic_L, a.magic_cd, a.magic_D, a.magic_G, a.local_counts, a.sync);
   const int nl = a.sh.n_logical, R = a.n_rep;
   const int tid = threadIdx.x;
   constexpr int nt = WAVES * kWave;
@@ -212,6 +218,9 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   if (pid < a.n_lp_workgroups) {
     // ------------------------------------------------------------ the LPs
     SolveArgs sa = a.solve;
+    fetch_arguments_now(sa.workload, sa.gw_out, sa.r2o, sa.phy2log, sa.avail, sa.result, sa.n_group, sa.G, sa.D, sa.C,
+                        sa.n_fixed, sa.n_experts, sa.step_rule, sa.n_steps, sa.n_units, sa.staged_stride, sa.tagged_result,
+                        sa.tagged_copies, sa.tagged_stride);
     const int first_lp = pid * kLpsPerWorkgroup;          // of this workgroup
     const int n_lps = min(kLpsPerWorkgroup, sa.n_units - first_lp);
     LPLB_PLAN_STAMP(0);
@@ -508,8 +517,13 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
       if (lane == 0) {
         if (!arrived)
           give_up(a, avail_state);
-        else if (slice == 0)
+        else if (slice == 0) {
           agent_store(a.sync + kGenAt, (gen + 1) & 0x3fffffff);   // every workgroup has read it by now
+          // From here on no workgroup of this launch waits for one that is not resident yet: tell the host, which
+          // then stops counting this launch against what the GPU can hold at once (a posted write to host memory).
+          if (a.arrived_word)
+            __hip_atomic_store(a.arrived_word, a.arrived_seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
         flags[0] = arrived;
       }
     }
@@ -697,14 +711,15 @@ static bool plan_lp_shape(int G, int D, int *gm, int *dm) {
 // does not see it.
 struct PlanSlot {
   hipStream_t stream = nullptr;
-  hipEvent_t done = nullptr;    // recorded behind the slot's latest one-launch plan (the library's own: the
-                                // stream handle may be stale by the time somebody asks)
+  int seq = 0;                  // number of the slot's latest launch outside a capture (what it writes when all
+                                // of its workgroups have arrived)
   float cost = 0.0f;            // share of the GPU's resident workgroups its launches take
   bool used = false, captured = false;
-  bool maybe_executing = false; // a launch was enqueued and its event has not been seen complete since
+  bool maybe_executing = false; // a launch was enqueued and has not been seen to have arrived since
 };
 struct PlanDevice {
   int *sync = nullptr;
+  int *arrived = nullptr;       // pinned host memory, one word per slot, written by the kernels (see PlanArgs)
   int n_cus = 0;
   PlanSlot slots[kSyncSlots];
 };
@@ -727,23 +742,26 @@ static int plan_device(PlanDevice **out) {
     LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&sync), HIP_SYMBOL(g_plan_sync)));
     d.n_cus = current_device_cu_count();
     LPLB_REQUIRE(d.n_cus > 0, LPLB_EHIP, "plan: cannot read the CU count of device %d", dev);
+    LPLB_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&d.arrived), kSyncSlots * sizeof(int), hipHostMallocDefault));
+    for (int i = 0; i < kSyncSlots; ++i)
+      d.arrived[i] = 0;
     d.sync = sync;
   }
   *out = &d;
   return LPLB_OK;
 }
 
-// May a launch of this slot still be executing?  Asks the runtime about the event recorded behind the
-// slot's latest plan; never waits and never touches the stream itself (other threads may be capturing
-// on it, or may have destroyed it).  may_ask = false (the calling stream is being captured: no queries
-// from inside a capture): what is not known to be over counts as executing.
-static bool slot_is_executing(PlanDevice &d, int i, bool may_ask) {
+// May a launch of this slot still need room on the GPU?  Once all workgroups of a launch have arrived none of
+// them waits for a workgroup that is not resident, and the launch says so in a word of pinned host memory:
+// looking at it asks nothing of the runtime, the stream (which other threads may be capturing on, or may
+// have destroyed) is not touched, and nothing waits.
+static bool slot_is_executing(PlanDevice &d, int i) {
   PlanSlot &s = d.slots[i];
   if (!s.used)
     return false;
   if (s.captured)
     return true;
-  if (s.maybe_executing && may_ask && s.done != nullptr && hipEventQuery(s.done) != hipErrorNotReady)
+  if (s.maybe_executing && __atomic_load_n(d.arrived + i, __ATOMIC_ACQUIRE) == s.seq)
     s.maybe_executing = false;
   return s.maybe_executing;
 }
@@ -759,13 +777,13 @@ static int admit_launch(PlanDevice &d, hipStream_t s, float cost, bool capturing
     if (!d.slots[i].used)
       slot = i;
   for (int i = 0; i < kSyncSlots && slot < 0; ++i)
-    if (!slot_is_executing(d, i, !capturing))
+    if (!slot_is_executing(d, i))
       slot = i;
   if (slot < 0)
     return -1;
   float executing = 0.0f;
   for (int i = 0; i < kSyncSlots; ++i)
-    if (i != slot && slot_is_executing(d, i, !capturing))
+    if (i != slot && slot_is_executing(d, i))
       executing += d.slots[i].cost;
   if (executing + cost > kResidencyBudget)
     return -1;
@@ -849,14 +867,14 @@ static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *don
   a.expected_slices = a.n_slices + g_fault_extra_slices.exchange(0);
   const int fault_polls = g_fault_max_polls.exchange(0);
   a.max_polls = fault_polls > 0 ? fault_polls : kDefaultMaxPolls;
-  // The event that says when this launch is over: the slot's own, made at its first launch outside a capture
-  // (a captured launch keeps its share of the GPU for good and needs none).
-  if (!capturing && ps.done == nullptr && hipEventCreateWithFlags(&ps.done, hipEventDisableTiming) != hipSuccess)
-    return fail(LPLB_EHIP, "plan: cannot create an event");
+  // (a captured launch keeps its share of the GPU for good and reports nothing)
+  if (!capturing) {
+    ps.seq = (ps.seq + 1) & 0x3fffffff;
+    a.arrived_word = d->arrived + slot;
+    a.arrived_seq = ps.seq;
+  }
   launch(kernel, dim3(n_workgroups), dim3(WAVES * kWave), lds, s, a);
-  hipError_t err = hipGetLastError();
-  if (err == hipSuccess && !capturing)
-    err = hipEventRecord(ps.done, s);
+  const hipError_t err = hipGetLastError();
   if (err != hipSuccess)
     return fail(LPLB_EHIP, "plan: launch failed: %s", hipGetErrorString(err));
   ps.maybe_executing = !capturing;
@@ -1019,6 +1037,11 @@ extern "C" int lplb_plan_sync_timeouts(int *count) {
     }
   }
   LPLB_HIP_TRY(hipDeviceSynchronize());
+  {
+    std::lock_guard<std::mutex> lock(g_plan_guard);   // nothing enqueued so far is still running
+    for (int slot = 0; slot < kSyncSlots; ++slot)
+      d->slots[slot].maybe_executing = false;
+  }
   return LPLB_OK;
 }
 
@@ -1135,7 +1158,8 @@ static __device__ __align__(256) int32_t scratch[kScratchInts];
 // outside a stream capture.  A call captured into a graph keeps the table for its stream for good.
 struct ScratchUse {
   int32_t *table = nullptr;
-  hipEvent_t done = nullptr;
+  int *finished = nullptr;   // pinned host memory: the number of the last call whose kernels have all ended
+  int seq = 0;               // number of the last call
   hipStream_t stream = nullptr;
   bool used = false, captured = false;
 };
@@ -1151,17 +1175,23 @@ static int scratch_of_current_device(ScratchUse **use) {
     int32_t *p = nullptr;
     LPLB_HIP_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
     LPLB_REQUIRE(p != nullptr, LPLB_EHIP, "plan_noalloc: no device address for the slice table");
-    LPLB_HIP_TRY(hipEventCreateWithFlags(&u.done, hipEventDisableTiming));
+    LPLB_HIP_TRY(hipHostMalloc(reinterpret_cast<void **>(&u.finished), sizeof(int), hipHostMallocDefault));
+    *u.finished = 0;
     u.table = p;
   }
   *use = &u;
   return LPLB_OK;
 }
 
-__global__ void copy_ints(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int n) {
+// The last kernel of a call: copies the batch's totals out (n may be 0) and says, in pinned host memory, that
+// every kernel of call number `seq` has ended (kernels of one stream end in the order they were enqueued).
+__global__ void copy_ints_and_report(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int n, int *finished,
+                                     int seq) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n)
     dst[i] = src[i];
+  if (i == 0 && finished)
+    __hip_atomic_store(finished, seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 } // namespace lplb
@@ -1210,8 +1240,7 @@ extern "C" int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
   if (rc != LPLB_OK)
     return rc;
   if (use->used && use->stream != s) {
-    // (from inside a capture the runtime is not asked: what is not known to be over counts as running)
-    const bool busy = use->captured || capturing || hipEventQuery(use->done) == hipErrorNotReady;
+    const bool busy = use->captured || __atomic_load_n(use->finished, __ATOMIC_ACQUIRE) != use->seq;
     LPLB_REQUIRE(!busy, LPLB_EBUSY,
                  "plan_noalloc: the built-in slice table is in use by a plan on another stream%s; wait for it, keep "
                  "such plans on one stream, or use lplb_plan with a workspace of your own",
@@ -1223,17 +1252,17 @@ extern "C" int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
   rc = plan_checked(idx, n_elements, global_counts, r2o, o2r, phy2log, n_group, group_size, dup_per_rank,
                     n_combined_experts, n_local_experts, n_blocks, table, global_workload, o_weight, avail_num, out,
                     physical_counts, step_rule, n_steps, stream);
-  if (rc == LPLB_OK && local_counts != nullptr) {
-    launch(copy_ints, dim3((unsigned)((n_logical + 255) / 256)), dim3(256), 0, s,
-           table + (int64_t)(n_blocks - 1) * n_logical, local_counts, (int)n_logical);
-    if (hipGetLastError() != hipSuccess)
-      rc = fail(LPLB_EHIP, "plan_noalloc: launch failed");
-  }
-  // whatever was enqueued may touch the table, also when a later step of the chain failed
+  // Whatever was enqueued may touch the table, also when a later step of the chain failed: the call is
+  // numbered and its last kernel reports the number (a captured call reports nothing: it keeps the table).
   use->used = true;
   use->stream = s;
   use->captured = use->captured || capturing;
-  if (!capturing && hipEventRecord(use->done, s) != hipSuccess && rc == LPLB_OK)
-    rc = fail(LPLB_EHIP, "plan_noalloc: cannot record an event");
+  if (!capturing)
+    use->seq = (use->seq + 1) & 0x3fffffff;
+  const int n_copy = rc == LPLB_OK && local_counts != nullptr ? (int)n_logical : 0;
+  launch(copy_ints_and_report, dim3((unsigned)((n_copy + 255) / 256 > 0 ? (n_copy + 255) / 256 : 1)), dim3(256), 0, s,
+         table + (int64_t)(n_blocks - 1) * n_logical, local_counts, n_copy, capturing ? nullptr : use->finished, use->seq);
+  if (hipGetLastError() != hipSuccess && rc == LPLB_OK)
+    rc = fail(LPLB_EHIP, "plan_noalloc: launch failed");
   return rc;
 }
