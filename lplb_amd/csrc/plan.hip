@@ -169,10 +169,6 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __shared__ int rep_of_edge_all[kLpsPerWorkgroup * kWave];
   __shared__ int flags[2];   // [0] the exchange of counts worked, [1] some share will not come
-  fetch_arguments_now(a.idx, a.n, a.per, a.n_slices, a.n_lp_workgroups, a.n_copies, a.n_arrival_copies, a.n_share_copies,
-                      a.expected_slices, a.max_polls, a.o2r, a.phy2log, a.rows, a.row_shift, a.totals, a.out,
-                      a.physical_counts, a.avail, a.sh.n_logical, a.sh.n_ranks, a.sh.G, a.sh.D, a.sh.C, a.sh.L, a.sh.P,
-                      a.n_rep, a.magic_L, a.magic_cd, a.magic_D, a.magic_G, a.local_counts, a.sync);
   const int nl = a.sh.n_logical, R = a.n_rep;
   const int tid = threadIdx.x;
   constexpr int nt = WAVES * kWave;
@@ -218,9 +214,6 @@ __global__ __launch_bounds__(WAVES *kWave, (GM * DM <= 16 && GM <= 8) ? 4 : 2) v
   if (pid < a.n_lp_workgroups) {
     // ------------------------------------------------------------ the LPs
     SolveArgs sa = a.solve;
-    fetch_arguments_now(sa.workload, sa.gw_out, sa.r2o, sa.phy2log, sa.avail, sa.result, sa.n_group, sa.G, sa.D, sa.C,
-                        sa.n_fixed, sa.n_experts, sa.step_rule, sa.n_steps, sa.n_units, sa.staged_stride, sa.tagged_result,
-                        sa.tagged_copies, sa.tagged_stride);
     const int first_lp = pid * kLpsPerWorkgroup;          // of this workgroup
     const int n_lps = min(kLpsPerWorkgroup, sa.n_units - first_lp);
     LPLB_PLAN_STAMP(0);

@@ -17,8 +17,6 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   __shared__ int rep_of_edge[kWave];
   __shared__ __attribute__((aligned(16))) double pivot_rows[2 * kWave];
   __shared__ __attribute__((aligned(16))) float tile[assembly_tile_floats<GM>()];
-  fetch_arguments_now(a.workload, a.gw_out, a.r2o, a.phy2log, a.avail, a.result, a.n_group, a.G, a.D, a.C, a.n_fixed,
-                      a.n_experts, a.step_rule, a.n_steps, a.n_units, a.staged_stride);
   if (blockIdx.x == 0 && threadIdx.x == 0)
     atomicAdd(a.avail, a.n_units);
   const int first_unit = blockIdx.x * ROWS;
