@@ -17,11 +17,6 @@ namespace lplb {
 
 constexpr int kLoadsInFlight = 4;   // 16-byte loads a thread issues before it consumes them
 
-__device__ inline void count_one(int32_t *hist, int64_t v, int n_experts) {
-  if (v >= 0 && v < n_experts)
-    atomicAdd(&hist[v], 1);
-}
-
 __global__ __launch_bounds__(1024) void slice_histogram(
     const int64_t *__restrict__ idx, int64_t n, int n_experts, int64_t per,
     int32_t *__restrict__ counts) {
@@ -29,10 +24,10 @@ __global__ __launch_bounds__(1024) void slice_histogram(
   fetch_arguments_now(idx, n, n_experts, per, counts);
   const int tid = threadIdx.x, nt = blockDim.x;
   const int p = blockIdx.x;
-  for (int e = tid; e < n_experts; e += nt)
-    hist[e] = 0;
-  __syncthreads();
-
+  auto count = [&](int64_t v) {
+    if ((uint64_t)v < (uint64_t)n_experts)
+      atomicAdd(&hist[(int)v], 1);
+  };
   const int64_t begin = slice_begin(n, per, p);
   const int64_t end = slice_begin(n, per, p + 1);
   // Pairs are loaded 16 bytes at a time.  Slices start on multiples of 256 indices,
@@ -41,24 +36,40 @@ __global__ __launch_bounds__(1024) void slice_histogram(
   // is counted alone.
   const int64_t head = (begin < end && (reinterpret_cast<uintptr_t>(idx + begin) & 8)) ? 1 : 0;
   const int64_t n_pairs = (end - begin - head) >> 1;
-  const longlong2 *pairs = reinterpret_cast<const longlong2 *>(idx + begin + head);
-  for (int64_t i0 = tid; i0 < n_pairs; i0 += (int64_t)nt * kLoadsInFlight) {
-    longlong2 v[kLoadsInFlight];
+  typedef long long i64x2 __attribute__((ext_vector_type(2)));
+  const i64x2 *pairs = reinterpret_cast<const i64x2 *>(idx + begin + head);
+  // the first batch of loads is on its way while the histogram is cleared
+  i64x2 first[kLoadsInFlight];
+#pragma unroll
+  for (int u = 0; u < kLoadsInFlight; ++u) {
+    const int64_t i = tid + (int64_t)u * nt;
+    first[u] = i < n_pairs ? __builtin_nontemporal_load(pairs + i) : i64x2{-1, -1};
+  }
+  for (int e = tid; e < n_experts; e += nt)
+    hist[e] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < kLoadsInFlight; ++u) {
+    count(first[u].x);
+    count(first[u].y);
+  }
+  for (int64_t i0 = tid + (int64_t)nt * kLoadsInFlight; i0 < n_pairs; i0 += (int64_t)nt * kLoadsInFlight) {
+    i64x2 v[kLoadsInFlight];
 #pragma unroll
     for (int u = 0; u < kLoadsInFlight; ++u) {
       const int64_t i = i0 + (int64_t)u * nt;
-      v[u] = i < n_pairs ? pairs[i] : longlong2{-1, -1};
+      v[u] = i < n_pairs ? __builtin_nontemporal_load(pairs + i) : i64x2{-1, -1};
     }
 #pragma unroll
     for (int u = 0; u < kLoadsInFlight; ++u) {
-      count_one(hist, v[u].x, n_experts);
-      count_one(hist, v[u].y, n_experts);
+      count(v[u].x);
+      count(v[u].y);
     }
   }
   if (tid == 0 && head)
-    count_one(hist, idx[begin], n_experts);
+    count(idx[begin]);
   if (tid == 0 && ((end - begin - head) & 1))
-    count_one(hist, idx[end - 1], n_experts);
+    count(idx[end - 1]);
   __syncthreads();
   int32_t *row = counts + (int64_t)p * n_experts;
   for (int e = tid; e < n_experts; e += nt)
@@ -124,9 +135,10 @@ int enqueue_count(const int64_t *idx, int64_t n_elements, int n_experts, int n_b
   LPLB_REQUIRE(lds <= 64 * 1024, LPLB_EUNSUPPORTED,
                "count_idx: n_experts=%d does not fit the LDS histogram", n_experts);
   const int64_t per = slice_len(n_elements, n_blocks);
-  // one 16-byte load per thread covers 2 indices: 256 threads for slices of up to
-  // 2048 indices (4 loads each), 1024 threads beyond that
-  const int threads = per <= 2 * 256 * kLoadsInFlight ? 256 : 1024;
+  // one 16-byte load per thread covers 2 indices; a thread has kLoadsInFlight of them under
+  // way, so a slice gets as many threads as cover it in one such batch, up to 1024
+  const int64_t batches = (per / 2 + kLoadsInFlight - 1) / kLoadsInFlight;
+  const int threads = batches <= 256 ? 256 : batches <= 512 ? 512 : 1024;
   launch_with_flags(slice_histogram, dim3(n_blocks), dim3(threads), lds, s,
                     any_order ? hipExtAnyOrderLaunch : 0u, idx, n_elements, n_experts, per, counts_by_block);
   LPLB_HIP_TRY(hipGetLastError());
