@@ -49,7 +49,7 @@ constexpr int kPlanLdsLimit = 160 * 1024 - 8 * 1024;   // dynamic LDS; the kerne
 // An LP workgroup's dynamic LDS starts with the areas its (up to four) LP waves work in, then
 // come the staged counts: per wave the pivot rows (2 * kWave doubles) and the assembly tile.
 constexpr size_t plan_lp_area_bytes(int gm) {
-  return 2 * kWave * sizeof(double) + (size_t)(gm >= kTileAssemblyMin ? gm * (gm + 4) + gm : 4) * sizeof(float);
+  return 2 * kWave * sizeof(double) + (size_t)assembly_tile_floats_of(gm) * sizeof(float);
 }
 constexpr int kDefaultMaxPolls = 1 << 22;   // a few seconds of polling before a wait gives up
 // LPs per LP workgroup: waves 0..3 of a workgroup sit on the CU's four SIMDs, and an LP

@@ -37,7 +37,9 @@ namespace lplb {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 // Group sizes from which the elimination takes its pivot rows from LDS (exact-fit variants; padded
 // ones from 16), and from which a lane's row of S is put together in LDS instead of registers.
-constexpr int kRowsFromLdsMin = 8, kTileAssemblyMin = 32;
+constexpr int kRowsFromLdsMin = 8, kTileAssemblyMin = 16;
+// With 16 or 32 ranks a wave has 4 or 2 lanes per rank: they share the rank's row of S (one LP per wave).
+constexpr bool rows_are_shared(int gm) { return gm == 16 || gm == 32; }
 
 struct SolveArgs {
   const int32_t *workload;   // [n_inst][n_experts]
@@ -183,10 +185,11 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, uint32_
                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// From 32 ranks on a lane's row of S is put together in LDS instead of registers: floats the
+// From 16 ranks on a lane's row of S is put together in LDS instead of registers: floats the
 // caller provides per wave (row i at i * (GM + 4), so that 16-byte reads of different lanes'
 // rows fall into different banks; then GM floats for a broadcast copy of v).
-template <int GM> constexpr int assembly_tile_floats() { return GM >= kTileAssemblyMin ? GM * (GM + 4) + GM : 4; }
+constexpr int assembly_tile_floats_of(int gm) { return gm >= kTileAssemblyMin ? gm * (gm + 4) + gm : 4; }
+template <int GM> constexpr int assembly_tile_floats() { return assembly_tile_floats_of(GM); }
 
 // GM, DM: register-array sizes (group size and replica slots rounded up).
 // EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
@@ -364,8 +367,24 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     for (int e = 0; e < NE; ++e)
       mask[e][c] = (oth[e] == c) ? -1.0f : 0.0f;
   }
+  // Shared rows (16 and 32 ranks, one LP per wave): for the elimination, wave lane l works on row
+  // l / TS of S and holds its columns k * TS + l % TS, k < KC.  Rows and the copy of v are laid out
+  // in LDS so that the columns of one lane are adjacent: column r at (r % TS) * KC + r / TS.
+  constexpr bool kShared = ROWS == 1 && rows_are_shared(GM);
+  constexpr int TS = kShared ? kWave / GM : 1, KC = GM / TS;
+  auto tile_pos = [](int r) { return (r % TS) * KC + r / TS; };
+  const int row_of_lane = wave_lane / TS, sub = wave_lane % TS;
   float *my_tile_row = tile + (lane < GM ? lane : GM - 1) * (GM + 4);
   float *v_copy = tile + GM * (GM + 4);
+  int oth_at[NE];
+#pragma unroll
+  for (int e = 0; e < NE; ++e)
+    oth_at[e] = tile_pos(oth[e]);
+  const int own_at = tile_pos(lane < GM ? lane : GM - 1);
+  const float *shared_row = tile + row_of_lane * (GM + 4) + sub * KC;   // my KC columns of my row ...
+  const float *shared_v = v_copy + sub * KC;                            // ... and v of those columns' ranks
+  const int v_of_row_at = tile_pos(row_of_lane);
+  const bool row_real = row_of_lane < G;
 
   LPLB_STAMP(3);
   // b_i = -(load of the experts that cannot move), minilp.cu:223-234
@@ -436,7 +455,8 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 
     if (step == 0) LPLB_STAMP(5);
     // Row `lane` of S and its right-hand side, fp64.
-    double S[GM];
+    double S[KC];
+    double rhs;
     const double dst = (double)st, dkv = (double)kappa * (double)v;
     const float st_col = is_rank ? st : 0.0f;
     if constexpr (kTileAssembly) {
@@ -450,15 +470,31 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 #pragma unroll
         for (int c4 = 0; c4 < GM / 4; ++c4)
           reinterpret_cast<f32x4 *>(my_tile_row)[c4] = zero;
-        v_copy[lane] = v;
+        v_copy[own_at] = v;
 #pragma unroll
         for (int e = 0; e < NE; ++e)
-          __hip_atomic_fetch_add(my_tile_row + oth[e], -lam_e[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-        __hip_atomic_fetch_add(my_tile_row + lane, lam_sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+          __hip_atomic_fetch_add(my_tile_row + oth_at[e], -lam_e[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+        __hip_atomic_fetch_add(my_tile_row + own_at, lam_sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if constexpr (kShared) {
+        // every lane of a row takes its KC columns; the row's own v comes from the copy as well
+        const double dkv_row = (double)kappa * (double)v_copy[v_of_row_at];
+        static_for<KC / 4>([&](auto k4c) {
+          constexpr int k4 = decltype(k4c)::value;
+          const f32x4 t4 = reinterpret_cast<const f32x4 *>(shared_row)[k4];
+          const f32x4 v4 = reinterpret_cast<const f32x4 *>(shared_v)[k4];
+          const float t[4] = {t4.x, t4.y, t4.z, t4.w}, vc[4] = {v4.x, v4.y, v4.z, v4.w};
+          static_for<4>([&](auto uu) {
+            constexpr int u = decltype(uu)::value, k = 4 * k4 + u;
+            const double base = (EXACT || (row_real && k * TS + sub < G)) ? dst : 0.0;
+            S[k] = __builtin_fma(dkv_row, (double)vc[u], base) + (double)t[u];
+          });
+        });
+        rhs = (EXACT || row_real) ? 1000.0 * dkv_row - dst : 0.0;
+      } else
       static_for<GM / 4>([&](auto c4c) {
         constexpr int c4 = decltype(c4c)::value;
         const f32x4 t4 = reinterpret_cast<const f32x4 *>(my_tile_row)[c4];
@@ -481,7 +517,8 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         S[c] = __builtin_fma(dkv, (double)lp_bcast<ROWS, c>(v), base) + (double)t;
       });
     }
-    double rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
+    if constexpr (!kShared)
+      rhs = (1000.0 * dkv - dst) * (EXACT ? 1.0 : row_on);
 
     if (step == 0) LPLB_STAMP(6);
     // Gauss-Jordan elimination of [S | rhs] by columns: lane i owns row i, column c
@@ -498,112 +535,213 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     // A lane's own multiple must be zero.  Rather than selecting on the chain (f is the
     // link between reciprocal and update), the lane's diagonal entry is cleared as soon
     // as it has been read as the pivot, one step ahead.
-    double my_pivot = 1.0;
-    double pivot = lp_bcast<ROWS, 0>(S[0]);
-    double rinv = rcp_f64(pivot);
-    // One LP per wave: the entries of pivot row c that the other rows need, S[c][c2] for
-    // c2 > c, are not fetched from lane c one by one (two v_readlane each).  The part of S
-    // that is still being eliminated stays symmetric (up to rounding), so they are also
-    // column c as it is spread over the lanes, S[c2][c] in lane c2: one LDS write of that
-    // register puts the whole row into LDS, and reads from a wave-uniform address hand two
-    // entries at a time to every lane.  LDS instructions do not take the vector ALU's issue
-    // slots, which are what bounds a lone wave.  Column c + 1 is final right after the first
-    // update of step c; it is written then, so the round trip through LDS overlaps the rest
-    // of step c and the reciprocal of the next pivot and is not part of the serial chain.
-    // Two buffers take turns, so a step's reads need not all be issued before the next write.
-    // (Measured per LP: 32 ranks 31.5 -> 22.2 us, 16 ranks 12.6 -> 11.2 us, 8 ranks 7.5 -> 7.2 us; four
-    // LPs per wave, each 16-lane row reading its own LP's column: 16384 LPs 30.9 -> 27.6 us.  The
-    // padded 8-rank variants keep the scalar broadcasts: inside the one-launch plan they have
-    // no register to spare at four waves per SIMD.)
-    constexpr bool kRowFromLds = (ROWS == 1 && (GM >= 16 || (GM >= kRowsFromLdsMin && EXACT))) || ROWS == 4;
-    constexpr int kChunk = 8;                       // columns per batch of LDS reads (GM is a multiple)
-    constexpr int kChunks = GM / kChunk;
-    constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
-    // chunk q of the row in buffer `parity`: columns 8 q .. 8 q + 7, four 16-byte reads
-    auto load_chunk = [&](int parity, int q, double (&buf)[kChunk]) {
-      const double2 *src = reinterpret_cast<const double2 *>(pivot_rows + parity * kWave + lane0 + q * kChunk);
+    float y;
+    if constexpr (kShared) {
+      // Shared rows.  The T lanes of row i all need the multiple f_i = S[i][c] / pivot: the lane that
+      // holds column c hands its entry to the others of its row with one quad-permute DPP move per
+      // half (rows are groups of 2 or 4 adjacent lanes).  That value is also what the row adds to
+      // the pivot row in LDS (S[c][i] = S[i][c]), stored part by part like the rows themselves, so
+      // a lane reads the entries under its own columns, two per 16-byte read, from one of TS
+      // addresses.  The pivot is read from, and the diagonal entry cleared in, the one lane that
+      // holds it, before the move: all lanes of row c then get f = 0.  A lane also updates columns
+      // left of the pivot that share a register index with live ones; nothing reads them again.
+      // The right-hand side and the pivots are kept by every lane of a row (same arithmetic in each),
+      // y is complete in a row's first lane.  Operation for operation this is the elimination
+      // below; only who holds what differs.
+      constexpr int kStride = KC + 2;                 // doubles between the parts of a pivot row (distinct banks)
+      constexpr int kPart = KC < 8 ? KC : 8;          // columns per batch of LDS reads
+      constexpr int kParts = KC / kPart;
+      static_assert(kParts <= 2 && TS * kStride <= kWave, "pivot rows are fetched in at most two batches");
+      const int publish_at = (row_of_lane % TS) * kStride + row_of_lane / TS;
+      const double *my_part = pivot_rows + sub * kStride;
+      auto share = [](auto jc, double v) {     // v of lane j of every group of TS lanes
+        constexpr int j = decltype(jc)::value;
+        constexpr int ctrl = TS == 4 ? j * 0x55 : (j == 0 ? 0xA0 : 0xF5);
+        int2 p = __builtin_bit_cast(int2, v);
+        p.x = __builtin_amdgcn_mov_dpp(p.x, ctrl, 0xF, 0xF, false);   // (every lane has a source: no old value)
+        p.y = __builtin_amdgcn_mov_dpp(p.y, ctrl, 0xF, 0xF, false);
+        return __builtin_bit_cast(double, p);
+      };
+      // columns [q * kPart, (q + 1) * kPart) of the pivot row in buffer `parity`, those from k_from on
+      auto load_part = [&](int parity, int q, int k_from, double (&buf)[kPart]) {
+        const double2 *src = reinterpret_cast<const double2 *>(my_part + parity * kWave + q * kPart);
 #pragma unroll
-      for (int j = 0; j < kChunk / 2; ++j) {
-        const double2 both = src[j];
-        buf[2 * j] = both.x;
-        buf[2 * j + 1] = both.y;
-      }
-      // The reads stay where they are written, ahead of their use: left alone, the compiler
-      // moves each one down to the instruction that needs it (fewer live registers) and the
-      // wave then waits out every LDS round trip.
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    // The first chunk a step needs is fetched during the step before, right after the column
-    // has been written (two sets of registers take turns).
-    double head[2][kChunk];
-    auto publish_column = [&](auto cc) {
-      constexpr int c = decltype(cc)::value;
-      if constexpr (kRowFromLds && c < GM) {
-        pivot_rows[(c % 2) * kWave + lane0 + lane] = S[c];   // (every lane writes: no branch; lanes >= GM are never read)
-        __builtin_amdgcn_wave_barrier();
-        if constexpr (c + 1 < GM)
-          load_chunk(c % 2, (c + 1) / kChunk, head[c % 2]);
-      }
-    };
-    publish_column(std::integral_constant<int, 0>{});
-    S[0] = lp_set_lane<ROWS, 0>(S[0], 0.0, lane);
-    static_for<GM>([&](auto cc) {
-      constexpr int c = decltype(cc)::value;
-      constexpr int q0 = (c + 1) / kChunk;          // chunk of column c + 1
-      double body[kBodySets][kChunk];
-      // S[c2] -= f * (row c)[c2]
-      auto clear = [&](auto c2c, double f) {
-        constexpr int c2 = decltype(c2c)::value;
-        if constexpr (c2 < GM) {
-          if constexpr (!kRowFromLds) {
-            S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
-          } else if constexpr (c2 / kChunk == q0) {
-            S[c2] = __builtin_fma(-f, head[c % 2][c2 % kChunk], S[c2]);
-          } else {
-            // entering a new chunk: fetch the one after it, and keep the compiler from pulling
-            // every later fetch up here (the rows would not fit the registers)
-            if constexpr (c2 % kChunk == 0 && kBodySets == 2) {
-              __builtin_amdgcn_sched_barrier(0);
-              if constexpr (c2 / kChunk + 1 < kChunks)
-                load_chunk(c % 2, c2 / kChunk + 1, body[(c2 / kChunk + 1) % kBodySets]);
-            }
-            S[c2] = __builtin_fma(-f, body[(c2 / kChunk) % kBodySets][c2 % kChunk], S[c2]);
+        for (int j = 0; j < kPart / 2; ++j)
+          if (q * kPart + 2 * j + 1 >= k_from) {
+            const double2 both = src[j];
+            buf[2 * j] = both.x;
+            buf[2 * j + 1] = both.y;
           }
+        __builtin_amdgcn_sched_barrier(0);   // the reads stay here, ahead of their use
+      };
+      double head[2][kPart];
+      double my_pivot = 1.0;
+      double pivot = readlane(S[0], 0);
+      double rinv = rcp_f64(pivot);
+      S[0] = lp_set_lane<1, 0>(S[0], 0.0, 0);
+      double col = share(std::integral_constant<int, 0>{}, S[0]);
+      pivot_rows[publish_at] = col;
+      __builtin_amdgcn_wave_barrier();
+      load_part(0, 0, 0, head[0]);
+      static_for<GM>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        constexpr int k1 = (c + 1) / TS;              // register of column c + 1, the first one still live
+        constexpr int q0 = k1 / kPart;
+        double body[kPart];
+        auto clear = [&](auto kc, double f) {
+          constexpr int k = decltype(kc)::value;
+          if constexpr (k < KC) {
+            if constexpr (k / kPart == q0)
+              S[k] = __builtin_fma(-f, head[c % 2][k % kPart], S[k]);
+            else
+              S[k] = __builtin_fma(-f, body[k % kPart], S[k]);
+          }
+        };
+        my_pivot = lp_set_lane<1, c * TS>(my_pivot, pivot, 0);
+        const double f = col * rinv;   // multiple of row c to subtract from my row (0 in row c)
+        double next_pivot = 1.0, estimate = 1.0, error = 0.0, next_col = 0.0;
+        if constexpr (q0 + 1 < kParts)
+          load_part(c % 2, q0 + 1, 0, body);
+        clear(std::integral_constant<int, k1>{}, f);
+        if constexpr (c + 1 < GM) {
+          constexpr int holder = (c + 1) * TS + (c + 1) % TS;   // lane with entry (c + 1, c + 1)
+          next_pivot = readlane(S[k1], holder);
+          estimate = __builtin_amdgcn_rcp(next_pivot);
+          S[k1] = lp_set_lane<1, holder>(S[k1], 0.0, 0);
+          next_col = share(std::integral_constant<int, (c + 1) % TS>{}, S[k1]);
+          pivot_rows[((c + 1) % 2) * kWave + publish_at] = next_col;
+          __builtin_amdgcn_wave_barrier();
+          constexpr int k1_next = (c + 2) / TS;
+          if constexpr (k1_next < KC)
+            load_part((c + 1) % 2, k1_next / kPart, k1_next, head[(c + 1) % 2]);
+        }
+        rhs = __builtin_fma(-f, readlane(rhs, c * TS), rhs);
+        clear(std::integral_constant<int, k1 + 1>{}, f);
+        if constexpr (c + 1 < GM)
+          error = __builtin_fma(-next_pivot, estimate, 1.0);
+        clear(std::integral_constant<int, k1 + 2>{}, f);
+        clear(std::integral_constant<int, k1 + 3>{}, f);
+        if constexpr (c + 1 < GM) {
+          rinv = __builtin_fma(error, estimate, estimate);   // = rcp_f64(next_pivot)
+          pivot = next_pivot;
+        }
+        static_for<(KC > k1 + 4 ? KC - k1 - 4 : 0)>([&](auto kk) {
+          clear(std::integral_constant<int, k1 + 4 + decltype(kk)::value>{}, f);
+        });
+        col = next_col;
+      });
+      if (step == 0) LPLB_STAMP(7);
+      const float y_of_row = (float)(rhs * rcp_f64(my_pivot));   // in the first lane of each row
+      const float y_mine = gather(y_of_row, (lane * TS) & (kWave - 1));
+      y = is_rank ? y_mine : 0.0f;
+    } else {
+      double my_pivot = 1.0;
+      double pivot = lp_bcast<ROWS, 0>(S[0]);
+      double rinv = rcp_f64(pivot);
+      // One LP per wave: the entries of pivot row c that the other rows need, S[c][c2] for
+      // c2 > c, are not fetched from lane c one by one (two v_readlane each).  The part of S
+      // that is still being eliminated stays symmetric (up to rounding), so they are also
+      // column c as it is spread over the lanes, S[c2][c] in lane c2: one LDS write of that
+      // register puts the whole row into LDS, and reads from a wave-uniform address hand two
+      // entries at a time to every lane.  LDS instructions do not take the vector ALU's issue
+      // slots, which are what bounds a lone wave.  Column c + 1 is final right after the first
+      // update of step c; it is written then, so the round trip through LDS overlaps the rest
+      // of step c and the reciprocal of the next pivot and is not part of the serial chain.
+      // Two buffers take turns, so a step's reads need not all be issued before the next write.
+      // (Measured per LP: 32 ranks 31.5 -> 22.2 us, 16 ranks 12.6 -> 11.2 us, 8 ranks 7.5 -> 7.2 us; four
+      // LPs per wave, each 16-lane row reading its own LP's column: 16384 LPs 30.9 -> 27.6 us.  The
+      // padded 8-rank variants keep the scalar broadcasts: inside the one-launch plan they have
+      // no register to spare at four waves per SIMD.)
+      constexpr bool kRowFromLds = (ROWS == 1 && (GM >= 16 || (GM >= kRowsFromLdsMin && EXACT))) || ROWS == 4;
+      constexpr int kChunk = 8;                       // columns per batch of LDS reads (GM is a multiple)
+      constexpr int kChunks = GM / kChunk;
+      constexpr int kBodySets = kChunks > 2 ? 2 : 1;  // chunks after a step's first are fetched one chunk ahead
+      // chunk q of the row in buffer `parity`: columns 8 q .. 8 q + 7, four 16-byte reads
+      auto load_chunk = [&](int parity, int q, double (&buf)[kChunk]) {
+        const double2 *src = reinterpret_cast<const double2 *>(pivot_rows + parity * kWave + lane0 + q * kChunk);
+#pragma unroll
+        for (int j = 0; j < kChunk / 2; ++j) {
+          const double2 both = src[j];
+          buf[2 * j] = both.x;
+          buf[2 * j + 1] = both.y;
+        }
+        // The reads stay where they are written, ahead of their use: left alone, the compiler
+        // moves each one down to the instruction that needs it (fewer live registers) and the
+        // wave then waits out every LDS round trip.
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // The first chunk a step needs is fetched during the step before, right after the column
+      // has been written (two sets of registers take turns).
+      double head[2][kChunk];
+      auto publish_column = [&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        if constexpr (kRowFromLds && c < GM) {
+          pivot_rows[(c % 2) * kWave + lane0 + lane] = S[c];   // (every lane writes: no branch; lanes >= GM are never read)
+          __builtin_amdgcn_wave_barrier();
+          if constexpr (c + 1 < GM)
+            load_chunk(c % 2, (c + 1) / kChunk, head[c % 2]);
         }
       };
-      my_pivot = lp_set_lane<ROWS, c>(my_pivot, pivot, lane);
-      const double f = S[c] * rinv;   // multiple of row c to subtract from my row (0 in lane c)
-      double next_pivot = 1.0, estimate = 1.0, error = 0.0;
-      if constexpr (kRowFromLds && q0 + 1 < kChunks)
-        load_chunk(c % 2, q0 + 1, body[(q0 + 1) % kBodySets]);
-      clear(std::integral_constant<int, c + 1>{}, f);
-      publish_column(std::integral_constant<int, c + 1>{});
-      if constexpr (c + 1 < GM) {
-        next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
-        estimate = __builtin_amdgcn_rcp(next_pivot);
-        S[c + 1] = lp_set_lane<ROWS, c + 1>(S[c + 1], 0.0, lane);
-      }
-      rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
-      clear(std::integral_constant<int, c + 2>{}, f);
-      if constexpr (c + 1 < GM)
-        error = __builtin_fma(-next_pivot, estimate, 1.0);
-      clear(std::integral_constant<int, c + 3>{}, f);
-      clear(std::integral_constant<int, c + 4>{}, f);
-      if constexpr (c + 1 < GM) {
-        rinv = __builtin_fma(error, estimate, estimate);   // = rcp_f64(next_pivot)
-        pivot = next_pivot;
-      }
-      static_for<(GM > c + 5 ? GM - c - 5 : 0)>([&](auto kk) {
-        constexpr int k = decltype(kk)::value;
-        // From 32 ranks on a row's broadcasts would fill the scalar registers if the
-        // compiler hoisted them all; fence them off in groups of eight columns.
-        if constexpr (!kRowFromLds && GM >= 32 && k % 8 == 0)
-          __builtin_amdgcn_sched_barrier(0);
-        clear(std::integral_constant<int, c + 5 + k>{}, f);
+      publish_column(std::integral_constant<int, 0>{});
+      S[0] = lp_set_lane<ROWS, 0>(S[0], 0.0, lane);
+      static_for<GM>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        constexpr int q0 = (c + 1) / kChunk;          // chunk of column c + 1
+        double body[kBodySets][kChunk];
+        // S[c2] -= f * (row c)[c2]
+        auto clear = [&](auto c2c, double f) {
+          constexpr int c2 = decltype(c2c)::value;
+          if constexpr (c2 < GM) {
+            if constexpr (!kRowFromLds) {
+              S[c2] = __builtin_fma(-f, lp_bcast<ROWS, c>(S[c2]), S[c2]);
+            } else if constexpr (c2 / kChunk == q0) {
+              S[c2] = __builtin_fma(-f, head[c % 2][c2 % kChunk], S[c2]);
+            } else {
+              // entering a new chunk: fetch the one after it, and keep the compiler from pulling
+              // every later fetch up here (the rows would not fit the registers)
+              if constexpr (c2 % kChunk == 0 && kBodySets == 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (c2 / kChunk + 1 < kChunks)
+                  load_chunk(c % 2, c2 / kChunk + 1, body[(c2 / kChunk + 1) % kBodySets]);
+              }
+              S[c2] = __builtin_fma(-f, body[(c2 / kChunk) % kBodySets][c2 % kChunk], S[c2]);
+            }
+          }
+        };
+        my_pivot = lp_set_lane<ROWS, c>(my_pivot, pivot, lane);
+        const double f = S[c] * rinv;   // multiple of row c to subtract from my row (0 in lane c)
+        double next_pivot = 1.0, estimate = 1.0, error = 0.0;
+        if constexpr (kRowFromLds && q0 + 1 < kChunks)
+          load_chunk(c % 2, q0 + 1, body[(q0 + 1) % kBodySets]);
+        clear(std::integral_constant<int, c + 1>{}, f);
+        publish_column(std::integral_constant<int, c + 1>{});
+        if constexpr (c + 1 < GM) {
+          next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
+          estimate = __builtin_amdgcn_rcp(next_pivot);
+          S[c + 1] = lp_set_lane<ROWS, c + 1>(S[c + 1], 0.0, lane);
+        }
+        rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
+        clear(std::integral_constant<int, c + 2>{}, f);
+        if constexpr (c + 1 < GM)
+          error = __builtin_fma(-next_pivot, estimate, 1.0);
+        clear(std::integral_constant<int, c + 3>{}, f);
+        clear(std::integral_constant<int, c + 4>{}, f);
+        if constexpr (c + 1 < GM) {
+          rinv = __builtin_fma(error, estimate, estimate);   // = rcp_f64(next_pivot)
+          pivot = next_pivot;
+        }
+        static_for<(GM > c + 5 ? GM - c - 5 : 0)>([&](auto kk) {
+          constexpr int k = decltype(kk)::value;
+          // From 32 ranks on a row's broadcasts would fill the scalar registers if the
+          // compiler hoisted them all; fence them off in groups of eight columns.
+          if constexpr (!kRowFromLds && GM >= 32 && k % 8 == 0)
+            __builtin_amdgcn_sched_barrier(0);
+          clear(std::integral_constant<int, c + 5 + k>{}, f);
+        });
       });
-    });
-    if (step == 0) LPLB_STAMP(7);
-    const float y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
+      if (step == 0) LPLB_STAMP(7);
+      y = is_rank ? (float)(rhs * rcp_f64(my_pivot)) : 0.0f;
+    }
 
     if (step == 0) LPLB_STAMP(8);
     // r = A^T w and the direction d = x (c - r); the edge part of w is
