@@ -560,6 +560,29 @@ def main() -> None:
             planner.run(idx, avail, n_sms)
         torch.cuda.synchronize()
         extras["planner_run_wall_us"] = round((time.perf_counter() - t) / 500 * 1e6, 2)
+        extras["planner_run_us_p50"] = round(pct(event_times_us(lambda: planner.run(idx, avail, n_sms), 1000, 100, torch), 50), 2)
+
+        # The same call on a Planner that was given a process group: histogram (lplb_count_idx), copy of the
+        # counts, all-reduce over the EP ranks, then LP and redirect as one plan on the summed counts.  One GPU:
+        # the all-reduce itself is left out (the stand-in group below is never handed to torch.distributed),
+        # everything around it runs as in a deployment.
+        class OneRankGroup:
+            def size(self):
+                return cfg.ep_size
+        grouped = Planner(torch.from_numpy(cfg.r2o), cfg.n_physical, cfg.n_logical, cfg.ep_size,
+                          group=OneRankGroup(), device=dev)
+        grouped.phy2log = phy2log
+        grouped.deep_ep_initialized = True     # "the counts are already reduced": skips torch.distributed.all_reduce
+        out_grouped = grouped.run(idx, avail, n_sms)
+        assert torch.equal(out_grouped, planner.run(idx, avail, n_sms)), "group path and one-launch path disagree"
+        extras["planner_run_with_group_us"] = round(
+            pct(event_times_us(lambda: grouped.run(idx, avail, n_sms), 1000, 100, torch), 50), 2)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(500):
+            grouped.run(idx, avail, n_sms)
+        torch.cuda.synchronize()
+        extras["planner_run_with_group_wall_us"] = round((time.perf_counter() - t) / 500 * 1e6, 2)
 
     # ------------------------------------------------------------ CPU baseline
     torch.set_num_threads(1)
