@@ -121,8 +121,9 @@ int lplb_count_idx(const int64_t *idx, int64_t n_elements, int n_experts,
  *   step_rule        LPLB_STEP_*; 0 reproduces the reference
  *   n_steps          number of affine-scaling steps; the reference uses 5
  *
- * Requires group_size * dup_per_rank <= 64 and dup_per_rank <= 8
- * (LPLB_EUNSUPPORTED otherwise).
+ * Requires group_size * dup_per_rank <= 128, group_size <= 64 and
+ * dup_per_rank <= 16 (LPLB_EUNSUPPORTED otherwise).  Up to 64 replica edges
+ * and 8 slots per rank a lane of the wave holds one edge; beyond that, two.
  */
 int lplb_solve(const int32_t *workload, float *global_workload,
                const int32_t *r2o, const int32_t *phy2log, int n_group,

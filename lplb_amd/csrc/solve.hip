@@ -11,16 +11,16 @@ namespace lplb {
 // the arithmetic).  So the first thread of the grid counts every LP of the launch as
 // feasible with one add, and a wave takes back the LPs of its own that failed -- rare,
 // and the sum is the same.
-template <int GM, int DM, bool EXACT, int ROWS>
+template <int GM, int DM, bool EXACT, int ROWS, int EPL>
 __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
   extern __shared__ float staged_all[];   // a.staged_stride floats per LP of this wave
-  __shared__ int rep_of_edge[kWave];
+  __shared__ int rep_of_edge[EPL * kWave];
   __shared__ __attribute__((aligned(16))) double pivot_rows[2 * kWave];
-  __shared__ __attribute__((aligned(16))) float tile[assembly_tile_floats<GM>()];
+  __shared__ __attribute__((aligned(16))) float tile[assembly_tile_floats<GM, EPL>()];
   if (blockIdx.x == 0 && threadIdx.x == 0)
     atomicAdd(a.avail, a.n_units);
   const int first_unit = blockIdx.x * ROWS;
-  const int n_ok = solve_lp<GM, DM, EXACT, ROWS>(a, first_unit, staged_all, rep_of_edge, pivot_rows, tile);
+  const int n_ok = solve_lp<GM, DM, EXACT, ROWS, EPL>(a, first_unit, staged_all, rep_of_edge, pivot_rows, tile);
   const int n_mine = min(max(a.n_units - first_unit, 0), ROWS);
   if (threadIdx.x == 0 && n_ok < n_mine)
     atomicAdd(a.avail, n_ok - n_mine);
@@ -34,11 +34,11 @@ __global__ __launch_bounds__(kWave) void solve_groups(SolveArgs a) {
 constexpr int kPackFrom = 1536;
 constexpr int kLdsLimit = 64 * 1024 - 2048;
 
-template <int GM, int DM, bool EXACT, int ROWS>
+template <int GM, int DM, bool EXACT, int ROWS, int EPL = 1>
 static void launch_variant(SolveArgs a, hipStream_t s) {
   const size_t lds = (size_t)ROWS * a.n_experts * sizeof(float);
   a.staged_stride = lds <= kLdsLimit ? a.n_experts : 0;
-  launch(solve_groups<GM, DM, EXACT, ROWS>, dim3((a.n_units + ROWS - 1) / ROWS), dim3(kWave),
+  launch(solve_groups<GM, DM, EXACT, ROWS, EPL>, dim3((a.n_units + ROWS - 1) / ROWS), dim3(kWave),
          a.staged_stride ? lds : 0, s, a);
 }
 
@@ -64,6 +64,18 @@ template <int GM, int DM> static void launch_solver(const SolveArgs &a, hipStrea
 
 static int dispatch(const SolveArgs &a, hipStream_t s) {
   const int G = a.G, D = a.D;
+  // 65 to 128 replica edges, or more than 8 slots per rank: two edges per lane, always the padded form (these shapes are rare, and one
+  // kernel per row of this list serves every (G, D) inside it).
+  if (G * D > kWave || D > 8) {
+#define LPLB_WIDE_CASE(GM, DM)                                                 \
+    if (G <= GM && D <= DM) {                                                  \
+      launch_variant<GM, DM, false, 1, 2>(a, s);                               \
+      return LPLB_OK;                                                          \
+    }
+    LPLB_WIDE_CASE(8, 16) LPLB_WIDE_CASE(16, 8) LPLB_WIDE_CASE(16, 16) LPLB_WIDE_CASE(32, 4) LPLB_WIDE_CASE(64, 2)
+#undef LPLB_WIDE_CASE
+    return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
+  }
 #define LPLB_CASE(GM, DM)                                                      \
   if (G <= GM && D <= DM) {                                                    \
     launch_solver<GM, DM>(a, s);                                               \
@@ -97,9 +109,9 @@ extern "C" int lplb_solve_batched(const int32_t *workloads, float *global_worklo
                n_steps);
   LPLB_REQUIRE(step_rule == LPLB_STEP_REFERENCE_WINDOW || step_rule == LPLB_STEP_FULL_MAX,
                LPLB_EINVAL, "solve: unknown step_rule %d", step_rule);
-  LPLB_REQUIRE(group_size * dup_per_rank <= kWave, LPLB_EUNSUPPORTED,
-               "solve: group_size*dup_per_rank=%d exceeds the 64 edges one wave holds",
-               group_size * dup_per_rank);
+  LPLB_REQUIRE(group_size * dup_per_rank <= 2 * kWave && group_size <= kWave && dup_per_rank <= 16, LPLB_EUNSUPPORTED,
+               "solve: group_size=%d dup_per_rank=%d: at most 128 replica edges (two per lane of a wave), 64 ranks, "
+               "16 slots per rank", group_size, dup_per_rank);
   const int64_t L = (int64_t)dup_per_rank * n_experts_per_var + n_experts_fixed;
   const int64_t n_experts = (int64_t)n_group * group_size * L;
   LPLB_REQUIRE(n_experts > 0 && n_experts <= (1 << 24) && (int64_t)n_instances * n_group <= INT32_MAX,

@@ -188,35 +188,43 @@ __device__ inline void store_share(float *p, unsigned long long *tagged, uint32_
 // From 16 ranks on a lane's row of S is put together in LDS instead of registers: floats the
 // caller provides per wave (row i at i * (GM + 4), so that 16-byte reads of different lanes'
 // rows fall into different banks; then GM floats for a broadcast copy of v).
-constexpr int assembly_tile_floats_of(int gm) { return gm >= kTileAssemblyMin ? gm * (gm + 4) + gm : 4; }
-template <int GM> constexpr int assembly_tile_floats() { return assembly_tile_floats_of(GM); }
+// (Also below 16 ranks when a lane holds two edges: the selectors would be 32 per column then.)
+constexpr int assembly_tile_floats_of(int gm, int epl = 1) {
+  return (gm >= kTileAssemblyMin || epl > 1) ? gm * (gm + 4) + gm : 4;
+}
+template <int GM, int EPL = 1> constexpr int assembly_tile_floats() { return assembly_tile_floats_of(GM, EPL); }
 
 // GM, DM: register-array sizes (group size and replica slots rounded up).
 // EXACT: the group is exactly GM x DM, so every loop bound is a compile-time
 // constant; otherwise rows and columns G..GM-1 of the normal-equation system are
 // padded with the identity, which keeps the factorisation free of branches.
 // ROWS: LPs per wave (1, or 4 when GM <= 16 and GM * DM <= 16).
+// EPL: replica edges per lane, 1 or 2 (ROWS == 1 only).  Edge j lives in lane j % 64, place j / 64;
+// groups with 65..128 edges take two places.  Everything per rank (the G x G system included) is
+// the same either way; what is per edge is done once per place, and a value of edge j is fetched
+// from place j / 64 of lane j % 64.
 //
 // Called by all 64 lanes of a wave; waves share nothing and never synchronise.
 //   first_unit     LP (instance * n_group + group) of the wave's first row
 //   staged_counts  LDS, ROWS * a.staged_stride floats (unused if the stride is 0)
-//   rep_of_edge    LDS, kWave ints
+//   rep_of_edge    LDS, EPL * kWave ints
 //   pivot_rows     LDS, 2 * kWave doubles of this wave, 16-byte aligned
-//   tile           LDS, assembly_tile_floats<GM>() floats of this wave, 16-byte aligned (32 ranks or more)
+//   tile           LDS, assembly_tile_floats<GM, EPL>() floats of this wave, 16-byte aligned
 // Returns how many of the wave's LPs passed the feasibility test (same value in
 // every lane); the caller adds it to a.avail.  -1: the counts the caller promised through
 // a.counts_ready never came; nothing was solved or stored.
-template <int GM, int DM, bool EXACT, int ROWS>
+template <int GM, int DM, bool EXACT, int ROWS, int EPL = 1>
 __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged_counts_of_wave,
                                int *rep_of_edge, double *pivot_rows, float *tile) {
   constexpr int WL = Layout<ROWS>::kWidth;   // lanes of one LP
   static_assert(ROWS == 1 || (ROWS == 4 && GM <= kRowLanes && GM * DM <= kRowLanes), "an LP must fit its lanes");
+  static_assert(EPL == 1 || (EPL == 2 && ROWS == 1), "two edges per lane only with one LP per wave");
   static_assert(GM % 8 == 0, "pivot rows are read from LDS eight columns at a time");
   constexpr int T = WL / GM;         // lanes that share the work of one rank's b_i
   constexpr int NE = 2 * DM;         // replica edges that touch one rank
   constexpr int KB = ROWS == 1 ? 4 : 16;   // fixed-expert counts a lane prefetches for b_i
   constexpr int WR = GM;             // lanes that can hold a rank
-  constexpr int WE = GM * DM < WL ? (GM * DM < 8 ? 8 : GM * DM) : WL;  // ... an edge
+  constexpr int WE = (GM * DM < WL && EPL == 1) ? (GM * DM < 8 ? 8 : GM * DM) : WL;  // ... an edge
   constexpr int KG = ROWS == 1 ? 4 : 16;   // normalised counts a lane prefetches for the output (and loop unrolling)
   const int wave_lane = threadIdx.x % kWave;
 
@@ -233,11 +241,27 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   const int grp = unit % a.n_group, inst = unit / a.n_group;
   float *staged_counts = staged_counts_of_wave + wave_lane / WL * a.staged_stride;
   auto gather = [&](auto v, int src) { return bpermute(v, lane0 + src); };
+  // value of edge `e` (v[place] of the lane that holds it)
+  auto gather_edge = [&](const auto (&v)[EPL], int e) {
+    if constexpr (EPL == 1) {
+      return bpermute(v[0], lane0 + e);
+    } else {
+      const auto lo = bpermute(v[0], e & (kWave - 1)), hi = bpermute(v[1], e & (kWave - 1));
+      return e < kWave ? lo : hi;
+    }
+  };
   const int32_t *__restrict__ wl = a.workload + (int64_t)inst * a.n_experts;
   const int32_t *__restrict__ p2l = a.phy2log + (int64_t)grp * G * P;
-  const bool is_edge = lane < n, is_rank = lane < G;
-  const int ek = is_edge ? lane / D : 0;   // original rank of my edge
-  const int ed = is_edge ? lane % D : 0;   // its replica slot
+  const bool is_rank = lane < G;
+  bool is_edge[EPL];
+  int ek[EPL], ed[EPL];   // original rank of my edge, its replica slot
+#pragma unroll
+  for (int p = 0; p < EPL; ++p) {
+    const int j = lane + p * kWave;
+    is_edge[p] = j < n;
+    ek[p] = is_edge[p] ? j / D : 0;
+    ed[p] = is_edge[p] ? j % D : 0;
+  }
   // When they fit, the counts are staged in LDS as floats, so that the gathers
   // through phy2log do not need a second round trip to global memory.
   const bool staged = a.staged_stride > 0;
@@ -250,7 +274,10 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   LPLB_STAMP(0);
   // ---- all global reads up front, as independent loads ----
   // (a) my edge's experts: raw count of the first, the rest in the loop below
-  const int e_first = (is_edge && C > 0) ? p2l[ek * P + ed] : -1;
+  int e_first[EPL];
+#pragma unroll
+  for (int p = 0; p < EPL; ++p)
+    e_first[p] = (is_edge[p] && C > 0) ? p2l[ek[p] * P + ed[p]] : -1;
   // (b) the experts of "my" rank that cannot move (T lanes share a rank)
   const int br = lane / T, bsub = lane % T;
   int fixed_e[KB];
@@ -308,7 +335,10 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     }
   }
   __builtin_amdgcn_wave_barrier();   // staged counts are visible to the whole wave
-  const float w_first = count_of(e_first);
+  float w_first[EPL];
+#pragma unroll
+  for (int p = 0; p < EPL; ++p)
+    w_first[p] = count_of(e_first[p]);
   float fixed_cnt[KB];
 #pragma unroll
   for (int u = 0; u < KB; ++u)
@@ -317,19 +347,26 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 
   LPLB_STAMP(1);
   // ---- per-edge constants (lane j < n): w_j, minilp.cu:203-221 ----
-  float w = is_edge && C > 0 ? w_first / wmax : 0.0f;
-  if (is_edge)
-    for (int c = 1; c < C; ++c)
-      w += count_of(p2l[ek * P + c * D + ed]) / wmax;
-  // rank that holds the copy of each edge: invert r2o through LDS
-  rep_of_edge[lane0 + lane] = ek;
+  float w[EPL];
+  int erep[EPL];
+#pragma unroll
+  for (int p = 0; p < EPL; ++p) {
+    w[p] = is_edge[p] && C > 0 ? w_first[p] / wmax : 0.0f;
+    if (is_edge[p])
+      for (int c = 1; c < C; ++c)
+        w[p] += count_of(p2l[ek[p] * P + c * D + ed[p]]) / wmax;
+    // rank that holds the copy of each edge: invert r2o through LDS
+    rep_of_edge[lane0 + lane + p * kWave] = ek[p];
+  }
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int d = 0; d < DM; ++d)
     if (is_rank && d < D)
       rep_of_edge[lane0 + r2o_row[d] * D + d] = lane;
   __builtin_amdgcn_wave_barrier();
-  const int erep = rep_of_edge[lane0 + lane];
+#pragma unroll
+  for (int p = 0; p < EPL; ++p)
+    erep[p] = rep_of_edge[lane0 + lane + p * kWave];
 
   LPLB_STAMP(2);
   // ---- per-rank constants (lane i < G) ----
@@ -346,8 +383,8 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     src[d] = on ? lane * D + d : 0;
     src[DM + d] = on ? r2o_row[d] * D + d : 0;
     // cross-lane reads stay outside lane-dependent conditions
-    const int other = gather(erep, src[d]);
-    const float w_own = gather(w, src[d]), w_copy = gather(w, src[DM + d]);
+    const int other = gather_edge(erep, src[d]);
+    const float w_own = gather_edge(w, src[d]), w_copy = gather_edge(w, src[DM + d]);
     oth[d] = on ? other : lane;
     oth[DM + d] = on ? r2o_row[d] : lane;
     w_e[d] = on ? w_own : 0.0f;
@@ -357,7 +394,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
   // of each edge's other end.
   // (From 32 ranks on the selectors alone would be 160 registers: there the row is put
   // together in LDS instead, see kTileAssembly below.)
-  constexpr bool kTileAssembly = ROWS == 1 && GM >= kTileAssemblyMin;
+  constexpr bool kTileAssembly = ROWS == 1 && (GM >= kTileAssemblyMin || EPL > 1);
   constexpr int GS = kTileAssembly ? 1 : GM;
   float mask[NE][GS], diag_mask[GS];
 #pragma unroll
@@ -421,29 +458,46 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
 
   LPLB_STAMP(4);
   // ---- affine scaling ----
-  float xo = 1.0f, xr = 1.0f, xs = 1.0f, xt = 1.0f, xM = 1.0f;
+  float xo[EPL], xr[EPL], xs = 1.0f, xt = 1.0f, xM = 1.0f;
+#pragma unroll
+  for (int p = 0; p < EPL; ++p)
+    xo[p] = xr[p] = 1.0f;
   float d_max = 0.0f;
   const int NV = 2 * n + G + 2;
   const int win_lo = a.step_rule == LPLB_STEP_REFERENCE_WINDOW ? (NV > 32 ? NV - 32 : 0) : 0;
   const bool with_zero = a.step_rule != LPLB_STEP_REFERENCE_WINDOW || NV < 32;
-  const bool win_o = is_edge && lane >= win_lo, win_r = is_edge && n + lane >= win_lo;
+  bool win_o[EPL], win_r[EPL];
+#pragma unroll
+  for (int p = 0; p < EPL; ++p) {
+    win_o[p] = is_edge[p] && lane + p * kWave >= win_lo;
+    win_r[p] = is_edge[p] && n + lane + p * kWave >= win_lo;
+  }
   const bool win_s = is_rank && 2 * n + lane >= win_lo;
   const double row_on = is_rank ? 1.0 : 0.0;
 
   for (int step = 0; step < a.n_steps; ++step) {
-    const float so = xo * xo, sr = xr * xr, ss = xs * xs, st = xt * xt, sM = xM * xM;
-    const float u = is_edge ? __builtin_amdgcn_rcpf(so + sr) : 0.0f;
-    const float wu = w * u;
-    const float ao = wu * so, ar = wu * sr;
-    const float lam = w * ao * sr;             // w^2 so sr / (so + sr)
-    const float sigma = lp_sum<ROWS, WE>(u);
+    const float ss = xs * xs, st = xt * xt, sM = xM * xM;
+    float so[EPL], sr[EPL], u[EPL], ao[EPL], ar[EPL], lam[EPL];
+    float u_all = 0.0f;
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) {
+      so[p] = xo[p] * xo[p];
+      sr[p] = xr[p] * xr[p];
+      u[p] = is_edge[p] ? __builtin_amdgcn_rcpf(so[p] + sr[p]) : 0.0f;
+      const float wu = w[p] * u[p];
+      ao[p] = wu * so[p];
+      ar[p] = wu * sr[p];
+      lam[p] = w[p] * ao[p] * sr[p];             // w^2 so sr / (so + sr)
+      u_all = p == 0 ? u[p] : u_all + u[p];
+    }
+    const float sigma = lp_sum<ROWS, WE>(u_all);
     const float kappa = sM * __builtin_amdgcn_rcpf(1.0f + sM * sigma);
 
     float q = 0.0f, lam_e[NE], lam_sum = ss;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float q_own = gather(ao, src[d]), q_copy = gather(ar, src[DM + d]);
-      const float l_own = gather(lam, src[d]), l_copy = gather(lam, src[DM + d]);
+      const float q_own = gather_edge(ao, src[d]), q_copy = gather_edge(ar, src[DM + d]);
+      const float l_own = gather_edge(lam, src[d]), l_copy = gather_edge(lam, src[DM + d]);
       // an inactive slot or a self-loop (oth == lane) contributes nothing to S;
       // an inactive slot contributes nothing to q either
       q += slot_on[d] ? q_own + q_copy : 0.0f;
@@ -746,16 +800,27 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     if (step == 0) LPLB_STAMP(8);
     // r = A^T w and the direction d = x (c - r); the edge part of w is
     // z = u (h - kappa u.h + kappa (m.y - 1000)), h = -B^T y.
-    const float yk = gather(y, ek), yrep = gather(y, erep);
-    const float hp = -w * (so * yk + sr * yrep);
+    float yk[EPL], yrep[EPL], hp[EPL];
+    float uhp_all = 0.0f;
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) {
+      yk[p] = gather(y, ek[p]);
+      yrep[p] = gather(y, erep[p]);
+      hp[p] = -w[p] * (so[p] * yk[p] + sr[p] * yrep[p]);
+      uhp_all = p == 0 ? u[p] * hp[p] : uhp_all + u[p] * hp[p];
+    }
     const float my = lp_sum<ROWS, WR>(m * y);
     const float sumy = lp_sum<ROWS, WR>(y);
-    const float uh = lp_sum<ROWS, WE>(u * hp);
+    const float uh = lp_sum<ROWS, WE>(uhp_all);
     const float shift = kappa * (my - 1000.0f) - kappa * uh;
-    const float z = u * (hp + shift);
     const float sumz = uh + shift * sigma;       // = sum of z over the edges
-    const float d_o = -xo * (w * yk + z);
-    const float d_r = -xr * (w * yrep + z);
+    float d_o[EPL], d_r[EPL];
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) {
+      const float z = u[p] * (hp[p] + shift);
+      d_o[p] = -xo[p] * (w[p] * yk[p] + z);
+      d_r[p] = -xr[p] * (w[p] * yrep[p] + z);
+    }
     const float d_s = -xs * y;
     const float d_t = xt * (1.0f + sumy);
     const float d_M = xM * (1000.0f - (my - sumz));
@@ -763,16 +828,22 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     if (step == 0) LPLB_STAMP(9);
     // Step length, minilp.cu:354-362.  NaN marks "not in the window".
     float cand = __builtin_nanf("");
-    cand = win_o ? fmaxf(cand, d_o) : cand;
-    cand = win_r ? fmaxf(cand, d_r) : cand;
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) {
+      cand = win_o[p] ? fmaxf(cand, d_o[p]) : cand;
+      cand = win_r[p] ? fmaxf(cand, d_r[p]) : cand;
+    }
     cand = win_s ? fmaxf(cand, d_s) : cand;
     cand = lane == 0 ? fmaxf(fmaxf(cand, d_t), d_M) : cand;
     d_max = lp_max<ROWS, WE>(cand);
     if (with_zero)
       d_max = fmaxf(d_max, 0.0f);
     const float alpha = (float)(0.999 / (double)d_max);
-    xo *= 1.0f - alpha * d_o;
-    xr *= 1.0f - alpha * d_r;
+#pragma unroll
+    for (int p = 0; p < EPL; ++p) {
+      xo[p] *= 1.0f - alpha * d_o[p];
+      xr[p] *= 1.0f - alpha * d_r[p];
+    }
     xs *= 1.0f - alpha * d_s;
     xt *= 1.0f - alpha * d_t;
     xM *= 1.0f - alpha * d_M;
@@ -786,20 +857,25 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
     float row = xs - xt + m * xM - b;
 #pragma unroll
     for (int d = 0; d < DM; ++d) {
-      const float a_o = gather(xo, src[d]), a_r = gather(xr, src[DM + d]);
+      const float a_o = gather_edge(xo, src[d]), a_r = gather_edge(xr, src[DM + d]);
       row += w_e[d] * a_o + w_e[DM + d] * a_r;
     }
     if (is_rank)
       res = fmaxf(res, fabsf(row));
-    if (is_edge)
-      res = fmaxf(res, fabsf(xo + xr - xM - 1.0f));
+#pragma unroll
+    for (int p = 0; p < EPL; ++p)
+      if (is_edge[p])
+        res = fmaxf(res, fabsf(xo[p] + xr[p] - xM - 1.0f));
     res = lp_max<ROWS, WE>(res);
   }
   const bool ok = (double)d_max < 0.1 && 0.0 <= (double)xM && (double)xM < 1e-4 &&
                   (double)res < 0.05;
   const int n_ok = __popcll(__ballot(lane == 0 && ok && unit_on));
-  if (is_edge && unit_on)
-    store_share(a.result, a.tagged_result, a.tag_valid, a.tagged_copies, a.tagged_stride, (int64_t)unit * n + lane, ok ? xo : 0.5f);
+#pragma unroll
+  for (int p = 0; p < EPL; ++p)
+    if (is_edge[p] && unit_on)
+      store_share(a.result, a.tagged_result, a.tag_valid, a.tagged_copies, a.tagged_stride,
+                  (int64_t)unit * n + lane + p * kWave, ok ? xo[p] : 0.5f);
   // Normalised counts of this group, for the caller.
   if (a.gw_out && unit_on) {
     float *gw = a.gw_out + (int64_t)inst * a.n_experts + grp * G * L;

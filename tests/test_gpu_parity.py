@@ -348,7 +348,11 @@ def test_solve_adversarial_distributions(cuda, topo):
 @pytest.mark.gpu
 @pytest.mark.parametrize("G,D,C,n_group", [(3, 1, 1, 1), (5, 2, 1, 3), (6, 3, 2, 1), (7, 4, 1, 2), (8, 8, 1, 1),
                                            (10, 6, 1, 1), (12, 2, 3, 2), (12, 5, 1, 1), (16, 4, 1, 1), (21, 3, 1, 1),
-                                           (24, 2, 1, 2), (32, 2, 2, 1), (40, 1, 1, 1), (64, 1, 1, 1)])
+                                           (24, 2, 1, 2), (32, 2, 2, 1), (40, 1, 1, 1), (64, 1, 1, 1),
+                                           # 65..128 replica edges or more than 8 slots per rank: two edges per lane
+                                           (16, 5, 1, 1), (12, 6, 1, 2), (8, 9, 1, 1), (8, 12, 1, 1), (10, 8, 2, 1),
+                                           (4, 12, 1, 1), (16, 8, 1, 1), (11, 9, 1, 1), (32, 3, 1, 1), (32, 4, 1, 1),
+                                           (24, 4, 1, 1), (64, 2, 1, 1), (48, 2, 1, 1), (8, 16, 1, 1)])
 def test_solve_random_topologies(cuda, G, D, C, n_group):
     """Replica topologies that are no named graph: every column of r2o is a random permutation
     (self-loops included), group sizes that do not fill the kernels' register arrays (padded
@@ -577,6 +581,41 @@ def test_run_matches_oracle_chain(cuda, cfg, mask):
     _compare_solve(shape, inp.phy2log, by_sm[-1], o_weight.cpu().numpy(), gw.cpu().numpy(), int(avail[0]))
     want = oracle.map_idx(inp.indices, o_weight.cpu().numpy(), by_sm, shape.o2r, inp.phy2log, shape.n_group,
                           shape.C, shape.P)
+    np.testing.assert_array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("g,shifts,n_group", [(16, [1, 2, 3, 4, 5], 1), (12, [1, 2, 3, 5, 7, 11], 2),
+                                             (8, [1, 2, 3, 4, 5, 6, 7, 1, 2], 1), (32, [1, 2, 16], 1)])
+def test_run_with_more_than_64_replica_edges(cuda, g, shifts, n_group):
+    """Groups with 65 to 128 replica edges (two edges per lane in the LP): Planner.run against the chain on
+    the CPU, as for the benchmark configurations."""
+    from lplb_amd.mapping import build_redundancy_mapping
+    rng = np.random.default_rng(g * 100 + len(shifts))
+    r2o = _shifted_ring(g, shifts)
+    d = len(shifts)
+    assert g * d > 64
+    ep = g * n_group
+    per_rank = d + 3
+    n_logical = ep * per_rank
+    shape = Shape(r2o, ep, n_logical, n_logical + d * ep)
+    hist = rng.integers(1, 1 << 20, size=n_logical).astype(np.int64)
+    phy2log, _, _ = build_redundancy_mapping(r2o, ep, n_logical, shape.n_physical, hist, n_nodes=1)
+    idx = rng.choice(n_logical, size=(6000, 4), p=rng.dirichlet(np.full(n_logical, 0.7))).astype(np.int64)
+    idx[rng.random(idx.shape) < 0.03] = -1
+    planner = Planner(torch.from_numpy(r2o), shape.n_physical, n_logical, ep)
+    planner.phy2log = dev(phy2log, cuda)
+    n_sms = 64
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+    d_idx = dev(idx, cuda)
+    out = planner.run(d_idx, avail, n_sms)
+    torch.cuda.synchronize()
+    by_sm = oracle.count_idx(idx, n_logical, n_sms)
+    local, by_sm_gpu = planner.count_workload(d_idx, n_sms)
+    np.testing.assert_array_equal(by_sm_gpu.cpu().numpy(), by_sm)
+    o_weight, gw = planner.solve_probs(local, torch.zeros(1, dtype=torch.int32, device=cuda))
+    _compare_solve(shape, phy2log, by_sm[-1], o_weight.cpu().numpy(), gw.cpu().numpy(), int(avail[0]))
+    want = oracle.map_idx(idx, o_weight.cpu().numpy(), by_sm, shape.o2r, phy2log, shape.n_group, shape.C, shape.P)
     np.testing.assert_array_equal(out.cpu().numpy(), want)
 
 
