@@ -120,6 +120,44 @@ class KernelTimer:
             self.hip.hipEventDestroy(b)
 
 
+def copy_sweep(lib, torch, dev) -> None:
+    """The library's copy kernel (what the redirect is compared with) at a range of sizes.  Every launch is
+    timed by its own begin/end timestamps; buffers rotate so that at least 512 MB of distinct lines pass
+    between two uses of the same one (fewer pairs, still more than the 256 MB last-level cache, at 128 MiB)."""
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for n_bytes in (16, 1 << 18, 1 << 20, 1 << 21, 1 << 22, 1 << 23, 3 << 22, 1 << 24, 1 << 25, 1 << 26, 1 << 27):
+        n_el = n_bytes // 8
+        n_pairs = int(min(18, max(3, -(-(512 << 20) // (2 * n_bytes)))))
+        src = [torch.randint(0, 256, (n_el,), dtype=torch.int64, device=dev) for _ in range(n_pairs)]
+        dst = [torch.empty_like(t) for t in src]
+        reps = 10
+        n = n_pairs * reps
+        arr = lambda ts: (ctypes.c_void_p * n)(*[ts[i % n_pairs].data_ptr() for i in range(n)])
+        a_src, a_dst = arr(src), arr(dst)
+        assert lib.lplb_copy_calibration_series(a_src, a_dst, n_el, n, None, None, stream) == 0   # warm-up pass
+        torch.cuda.synchronize()
+        timer = KernelTimer(lib, n)
+        starts, stops = timer.take(n)
+        assert lib.lplb_copy_calibration_series(a_src, a_dst, n_el, n, starts, stops, stream) == 0, lib.lplb_last_error()
+        us = timer.times_us(torch)
+        timer.close()
+        assert torch.equal(dst[0], src[0])
+        rows.append({"bytes_each_way": n_bytes, "buffer_pairs": n_pairs, "launches": n,
+                     "avg_us": round(float(us.mean()), 2), "p50_us": round(pct(us, 50), 2),
+                     "min_us": round(float(us.min()), 2),
+                     "GBs_avg": round(2 * n_bytes / (float(us.mean()) * 1e-6) / 1e9, 1),
+                     "frac_of_peak_avg": round(2 * n_bytes / (float(us.mean()) * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+        del src, dst
+    # time = fixed + bytes / rate, fitted over the sizes from 1 MiB up
+    big = [r for r in rows if r["bytes_each_way"] >= 1 << 20]
+    x = np.array([2.0 * r["bytes_each_way"] for r in big])
+    y = np.array([r["avg_us"] for r in big])
+    slope, fixed = np.polyfit(x, y, 1)
+    print(json.dumps({"copy_sweep": rows, "fit_from_1MiB": {"fixed_us": round(float(fixed), 2),
+                                                           "GBs": round(1e-3 / float(slope), 1)}}))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +170,9 @@ def main() -> None:
     ap.add_argument("--roofline-reps", type=int, default=20, help="passes over the rotating buffers")
     ap.add_argument("--solver-only", action="store_true",
                     help="only 50 single and 10 batched (2048) LP solves at the plan's shape (for counter collection)")
+    ap.add_argument("--copy-sweep", action="store_true",
+                    help="only the copy kernel, from 16 bytes to 128 MiB per direction: the fixed cost of a launch "
+                         "and what a streaming kernel of the sweep's size can reach on this box")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the plan; a run with --gpus > 1 is not supported "
@@ -153,6 +194,10 @@ def main() -> None:
 
     def to_dev(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    if args.copy_sweep:
+        copy_sweep(load(), torch, dev)
+        return
 
     # ------------------------------------------------------------------ inputs
     inp = synth.make_inputs("v3_ep8_cube")

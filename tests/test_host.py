@@ -237,8 +237,10 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.lplb_count_idx(p, -1, 8, 4, p, None) == 1
     assert lib.lplb_count_idx(p, 4, 8, 4, None, None) == 1
     assert lib.lplb_count_idx(p, 4, 1 << 20, 4, p, None) == 2           # histogram does not fit LDS
-    assert lib.lplb_solve(p, p, p, p, 1, 8, 16, 1, 2, p, p, 0, 5, None) == 2   # 128 edges > one wave
-    assert b"64 edges" in lib.lplb_last_error()
+    assert lib.lplb_solve(p, p, p, p, 1, 16, 9, 1, 2, p, p, 0, 5, None) == 2   # 144 edges > two per lane of a wave
+    assert b"128 replica edges" in lib.lplb_last_error()
+    assert lib.lplb_solve(p, p, p, p, 1, 4, 17, 1, 2, p, p, 0, 5, None) == 2   # more than 16 slots per rank
+    assert lib.lplb_solve(p, p, p, p, 1, 65, 1, 1, 2, p, p, 0, 5, None) == 2   # more ranks than lanes
     assert lib.lplb_solve(p, p, p, p, 1, 8, 2, 1, 2, p, p, 7, 5, None) == 1    # unknown step rule
     assert lib.lplb_solve(p, None, p, p, 1, 8, 2, 1, 2, p, p, 0, 5, None) == 1
     assert lib.lplb_solve_batched(p, None, p, p, 0, 1, 8, 2, 1, 2, p, p, 0, 5, None) == 1
