@@ -597,14 +597,20 @@ def main() -> None:
         from lplb_amd import Planner
         planner = Planner(torch.from_numpy(cfg.r2o), cfg.n_physical, cfg.n_logical, cfg.ep_size, device=dev)
         planner.phy2log = phy2log
-        for _ in range(50):
-            planner.run(idx, avail, n_sms)
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(500):
-            planner.run(idx, avail, n_sms)
-        torch.cuda.synchronize()
-        extras["planner_run_wall_us"] = round((time.perf_counter() - t) / 500 * 1e6, 2)
+
+        def wall_us_per_call(fn):
+            """Median over five runs of 500 calls, each ended by a device sync (the first run after a pause
+            reads up to twice the others)."""
+            runs = []
+            for _ in range(6):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(500):
+                    fn()
+                torch.cuda.synchronize()
+                runs.append((time.perf_counter() - t) / 500 * 1e6)
+            return round(float(np.median(runs[1:])), 2)
+        extras["planner_run_wall_us"] = wall_us_per_call(lambda: planner.run(idx, avail, n_sms))
         extras["planner_run_us_p50"] = round(pct(event_times_us(lambda: planner.run(idx, avail, n_sms), 1000, 100, torch), 50), 2)
 
         # The same call on a Planner that was given a process group: histogram (lplb_count_idx), copy of the
@@ -622,12 +628,7 @@ def main() -> None:
         assert torch.equal(out_grouped, planner.run(idx, avail, n_sms)), "group path and one-launch path disagree"
         extras["planner_run_with_group_us"] = round(
             pct(event_times_us(lambda: grouped.run(idx, avail, n_sms), 1000, 100, torch), 50), 2)
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(500):
-            grouped.run(idx, avail, n_sms)
-        torch.cuda.synchronize()
-        extras["planner_run_with_group_wall_us"] = round((time.perf_counter() - t) / 500 * 1e6, 2)
+        extras["planner_run_with_group_wall_us"] = wall_us_per_call(lambda: grouped.run(idx, avail, n_sms))
 
     # ------------------------------------------------------------ CPU baseline
     torch.set_num_threads(1)

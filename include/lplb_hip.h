@@ -241,8 +241,10 @@ int lplb_map_idx_prepared(const int64_t *idx, const float *o_weight,
  * The one-launch form: its workgroups wait for each other, so the whole grid has to be
  * resident on the GPU.  The library admits a launch only if the grid fits (worked out
  * from the kernel's registers and LDS) beside the one-launch plans that are still executing, of which it keeps
- * track per stream (eight streams per device at a time; it asks the runtime whether
- * those streams still have work pending, it never waits); otherwise the call runs the
+ * track per stream (eight streams per device at a time; every launch writes its number
+ * into pinned host memory once all its workgroups have arrived, and the library looks at
+ * those words: it never waits and never hands a stream of the caller's to the runtime
+ * after the call that brought it); otherwise the call runs the
  * chain, with identical results.  A plan captured into a graph keeps its share of the GPU reserved
  * from then on (its replays are invisible to the library).  Launches on one stream never overlap; the exception the
  * library cannot see is a graph captured on one stream and replayed concurrently on
