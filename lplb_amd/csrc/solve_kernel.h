@@ -147,6 +147,19 @@ template <int ROWS, int LANE> __device__ inline double lp_set_lane(double old, d
     return lane == LANE ? v : old;
   }
 }
+// `old` with lane LANE of this LP's lanes made zero.  One LP per wave: only the high word is
+// cleared (one v_writelane instead of two, and it sits in the chain from one pivot to the next).
+// What is left is a denormal below 2^-1022 (or zero where denormals are flushed): as a multiplier
+// in S[k] -= f * x it changes no entry that is not itself that small.
+template <int ROWS, int LANE> __device__ inline double lp_clear_lane(double old, int lane) {
+  if constexpr (ROWS == 1) {
+    int2 o = __builtin_bit_cast(int2, old);
+    asm("v_writelane_b32 %0, 0, %1" : "+v"(o.y) : "n"(LANE));
+    return __builtin_bit_cast(double, o);
+  } else {
+    return lane == LANE ? 0.0 : old;
+  }
+}
 // Reductions over the first W lanes of this LP (W <= 16 when ROWS == 4).
 template <int ROWS, int W> __device__ inline float lp_sum(float v) {
   if constexpr (ROWS == 1) {
@@ -632,7 +645,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
       double my_pivot = 1.0;
       double pivot = readlane(S[0], 0);
       double rinv = rcp_f64(pivot);
-      S[0] = lp_set_lane<1, 0>(S[0], 0.0, 0);
+      S[0] = lp_clear_lane<1, 0>(S[0], 0);
       double col = share(std::integral_constant<int, 0>{}, S[0]);
       pivot_rows[publish_at] = col;
       __builtin_amdgcn_wave_barrier();
@@ -661,7 +674,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
           constexpr int holder = (c + 1) * TS + (c + 1) % TS;   // lane with entry (c + 1, c + 1)
           next_pivot = readlane(S[k1], holder);
           estimate = __builtin_amdgcn_rcp(next_pivot);
-          S[k1] = lp_set_lane<1, holder>(S[k1], 0.0, 0);
+          S[k1] = lp_clear_lane<1, holder>(S[k1], 0);
           next_col = share(std::integral_constant<int, (c + 1) % TS>{}, S[k1]);
           pivot_rows[((c + 1) % 2) * kWave + publish_at] = next_col;
           __builtin_amdgcn_wave_barrier();
@@ -737,7 +750,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         }
       };
       publish_column(std::integral_constant<int, 0>{});
-      S[0] = lp_set_lane<ROWS, 0>(S[0], 0.0, lane);
+      S[0] = lp_clear_lane<ROWS, 0>(S[0], lane);
       static_for<GM>([&](auto cc) {
         constexpr int c = decltype(cc)::value;
         constexpr int q0 = (c + 1) / kChunk;          // chunk of column c + 1
@@ -772,7 +785,7 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
         if constexpr (c + 1 < GM) {
           next_pivot = lp_bcast<ROWS, c + 1>(S[c + 1]);
           estimate = __builtin_amdgcn_rcp(next_pivot);
-          S[c + 1] = lp_set_lane<ROWS, c + 1>(S[c + 1], 0.0, lane);
+          S[c + 1] = lp_clear_lane<ROWS, c + 1>(S[c + 1], lane);
         }
         rhs = __builtin_fma(-f, lp_bcast<ROWS, c>(rhs), rhs);
         clear(std::integral_constant<int, c + 2>{}, f);
