@@ -24,11 +24,13 @@
 // rank-one terms -- with right-hand side -t^2 1 + 1000 kappa v, where
 //     E_j = x_o^2 + x_r^2, u_j = 1/E_j, lambda_j = w_j^2 x_o^2 x_r^2 u_j,
 //     kappa = x_M^2 / (1 + x_M^2 sum u), q = B u, v = m + q.
-// Lane i of the wave owns rank i and row i of S, lane j owns edge j.  S is
-// assembled and [S | rhs] reduced by Gauss-Jordan elimination (pivots and pivot-row
-// entries broadcast with v_readlane, every lane updating its own row) in fp64: the
-// system is tiny, and fp64 here removes the 1e-4..1e-3 rounding scatter a 32-bit
-// factorisation shows on nearly balanced loads.  Everything else is fp32.
+// Lane i of the wave owns rank i, lane j owns edge j (two edges per lane beyond 64).  S is
+// assembled and [S | rhs] reduced by Gauss-Jordan elimination in fp64: the system is tiny,
+// and fp64 here removes the 1e-4..1e-3 rounding scatter a 32-bit factorisation shows on
+// nearly balanced loads.  Everything else is fp32.  For the elimination, lane i holds row i
+// of S (8 and 64 ranks, and four LPs per wave), or the 4 or 2 lanes per rank that a wave has
+// at 16 or 32 ranks share the row; pivots are broadcast with v_readlane, the pivot row's
+// entries with v_readlane or through LDS, and every lane updates what it holds.
 #pragma once
 #include "common.h"
 
@@ -612,9 +614,9 @@ __device__ inline int solve_lp(const SolveArgs &a, int first_unit, float *staged
       // addresses.  The pivot is read from, and the diagonal entry cleared in, the one lane that
       // holds it, before the move: all lanes of row c then get f = 0.  A lane also updates columns
       // left of the pivot that share a register index with live ones; nothing reads them again.
-      // The right-hand side and the pivots are kept by every lane of a row (same arithmetic in each),
-      // y is complete in a row's first lane.  Operation for operation this is the elimination
-      // below; only who holds what differs.
+      // The right-hand side is kept by every lane of a row (same arithmetic in each), the pivot of
+      // a row by its first lane, where y is complete.  Operation for operation this is the
+      // elimination below; only who holds what differs.
       constexpr int kStride = KC + 2;                 // doubles between the parts of a pivot row (distinct banks)
       constexpr int kPart = KC < 8 ? KC : 8;          // columns per batch of LDS reads
       constexpr int kParts = KC / kPart;
