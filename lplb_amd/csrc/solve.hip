@@ -72,7 +72,8 @@ static int dispatch(const SolveArgs &a, hipStream_t s) {
       launch_variant<GM, DM, false, 1, 2>(a, s);                               \
       return LPLB_OK;                                                          \
     }
-    LPLB_WIDE_CASE(8, 16) LPLB_WIDE_CASE(16, 8) LPLB_WIDE_CASE(16, 16) LPLB_WIDE_CASE(32, 4) LPLB_WIDE_CASE(64, 2)
+    LPLB_WIDE_CASE(8, 16) LPLB_WIDE_CASE(16, 8) LPLB_WIDE_CASE(16, 16) LPLB_WIDE_CASE(32, 4) LPLB_WIDE_CASE(32, 8)
+    LPLB_WIDE_CASE(64, 2) LPLB_WIDE_CASE(64, 4)
 #undef LPLB_WIDE_CASE
     return fail(LPLB_EUNSUPPORTED, "solve: group_size=%d dup_per_rank=%d has no kernel", G, D);
   }

@@ -352,7 +352,8 @@ def test_solve_adversarial_distributions(cuda, topo):
                                            # 65..128 replica edges or more than 8 slots per rank: two edges per lane
                                            (16, 5, 1, 1), (12, 6, 1, 2), (8, 9, 1, 1), (8, 12, 1, 1), (10, 8, 2, 1),
                                            (4, 12, 1, 1), (16, 8, 1, 1), (11, 9, 1, 1), (32, 3, 1, 1), (32, 4, 1, 1),
-                                           (24, 4, 1, 1), (64, 2, 1, 1), (48, 2, 1, 1), (8, 16, 1, 1)])
+                                           (24, 4, 1, 1), (64, 2, 1, 1), (48, 2, 1, 1), (8, 16, 1, 1), (20, 6, 1, 1), (17, 7, 1, 1),
+                                           (33, 3, 1, 1), (42, 3, 1, 1)])
 def test_solve_random_topologies(cuda, G, D, C, n_group):
     """Replica topologies that are no named graph: every column of r2o is a random permutation
     (self-loops included), group sizes that do not fill the kernels' register arrays (padded
