@@ -234,8 +234,10 @@ class Planner:
         table = ws.get("group_counts")
         if table is None or table.device != idx.device:
             table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32, device=idx.device)
-        local_workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
-        workload = local_workload.clone()
+        # (The reference copies the counts before it reduces them, lplb/planner.py:215, because its redirect
+        # reads the same table afterwards.  This table is not read again -- the plan counts its slices
+        # itself -- so the sum may replace its last row.)
+        workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
         if not self.deep_ep_initialized:
             torch.distributed.all_reduce(workload, group=self.ep_group)
         out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,
