@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 5
+#define LPLB_ABI_VERSION 6
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -101,6 +101,20 @@ int lplb_map_idx_prepared_series(const int64_t *const *idx, const float *o_weigh
  */
 int lplb_count_idx(const int64_t *idx, int64_t n_elements, int n_experts,
                    int n_blocks, int32_t *counts_by_block, lplb_stream_t stream);
+
+/*
+ * This GPU's tokens per expert and nothing else (the last row of lplb_count_idx's
+ * table), in one kernel launch.  No counterpart in the reference: it serves
+ * Planner.run with a process group, which needs the counts for the all-reduce
+ * ahead of the plan and no table (lplb/planner.py:209-216 gets them from count_idx).
+ * Every workgroup reads the whole batch, so this is for short batches:
+ * n_elements <= 131072 and n_experts <= 1024, LPLB_EUNSUPPORTED beyond (callers
+ * then use lplb_count_idx).
+ *
+ *   totals           int32 [n_experts], out
+ */
+int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_experts,
+                      int32_t *totals, lplb_stream_t stream);
 
 /*
  * Builds and solves one LP per EP group: minimise the maximum per-rank load by

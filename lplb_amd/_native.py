@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1
@@ -37,6 +37,7 @@ _SIGNATURES = {
     "lplb_copy_calibration_series": (_i, [_vp, _vp, _i64, _i, _vp, _vp, _vp]),
     "lplb_map_idx_prepared_series": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
+    "lplb_count_totals": (_i, [_vp, _i64, _i, _vp, _vp]),
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
@@ -259,6 +260,19 @@ class CompiledSolver:
         _check(self.lib.lplb_count_idx(idx.data_ptr(), idx.numel(), self.n_experts, n_sms, out.data_ptr(),
                                        _stream(idx)))
         return out[-1], out
+
+    def count_totals(self, idx: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """This GPU's tokens per logical expert (what count_idx returns first) without the table per slice, in
+        one kernel launch; short batches only (UnsupportedShape beyond 131072 indices or 1024 experts).  No
+        counterpart in the reference."""
+        _require(idx.dtype == torch.int64 and idx.is_cuda and idx.is_contiguous(), "idx is a contiguous int64 GPU tensor")
+        if out is None:
+            out = torch.empty(self.n_experts, dtype=torch.int32, device=idx.device)
+        else:
+            _require(out.dtype == torch.int32 and out.is_cuda and out.is_contiguous() and out.numel() == self.n_experts,
+                     "out: int32 [n_experts], contiguous, on the GPU")
+        _check(self.lib.lplb_count_totals(idx.data_ptr(), idx.numel(), self.n_experts, out.data_ptr(), _stream(idx)))
+        return out
 
     # -- csrc/plugin.cpp:602-660 -------------------------------------------------
     def map_idx(self, mapping_idx: torch.Tensor, o_weight: torch.Tensor, local_workload_split_by_sm: torch.Tensor,

@@ -126,6 +126,79 @@ __global__ __launch_bounds__(kScanBands *kScanCols) void prefix_over_slices(
   }
 }
 
+// ---- totals only, for short batches: one launch, nothing shared between workgroups ----
+// A workgroup owns kOwned experts and reads the whole batch; what it counts is final, so there is no
+// second kernel, no atomic between workgroups and nothing to clear.  Every workgroup pulls all n indices
+// through its CU (64 bytes per clock), which bounds the batch this pays for: 65536 indices take about as
+// long as the launch itself, against two launches for histogram and scan.  A lane keeps four counters;
+// the values of a batch of loads are first added up in one register, a byte per owned expert.
+constexpr int kOwned = 4;
+constexpr int64_t kTotalsMaxIndices = 1 << 17;   // per call; beyond, the two-kernel form is faster
+constexpr int kTotalsMaxExperts = 1024;
+
+__global__ __launch_bounds__(1024) void expert_totals(const int64_t *__restrict__ idx, int64_t n, int n_experts,
+                                                      int32_t *__restrict__ totals) {
+  __shared__ int32_t per_wave[16][kOwned];
+  fetch_arguments_now(idx, n, n_experts, totals);
+  typedef long long i64x2 __attribute__((ext_vector_type(2)));
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t base = (int64_t)blockIdx.x * kOwned;
+  // one byte per owned expert: 1 << (8 * (v - base)) for a value this workgroup owns, else 0
+  auto key = [&](int64_t v) -> uint32_t {
+    const uint64_t rel = (uint64_t)(v - base);
+    return rel < (uint64_t)kOwned && v < n_experts ? 1u << (8 * (uint32_t)rel) : 0u;
+  };
+  const int64_t head = (n > 0 && (reinterpret_cast<uintptr_t>(idx) & 8)) ? 1 : 0;   // (see slice_histogram)
+  const int64_t n_pairs = (n - head) >> 1;
+  const i64x2 *pairs = reinterpret_cast<const i64x2 *>(idx + head);
+  uint32_t mine[kOwned] = {};
+  for (int64_t i0 = tid; i0 < n_pairs; i0 += (int64_t)nt * kLoadsInFlight) {
+    i64x2 v[kLoadsInFlight];
+#pragma unroll
+    for (int u = 0; u < kLoadsInFlight; ++u) {
+      const int64_t i = i0 + (int64_t)u * nt;
+      v[u] = i < n_pairs ? pairs[i] : i64x2{-1, -1};
+    }
+    uint32_t packed = 0;   // at most 2 * kLoadsInFlight per byte
+#pragma unroll
+    for (int u = 0; u < kLoadsInFlight; ++u)
+      packed += key(v[u].x) + key(v[u].y);
+#pragma unroll
+    for (int k = 0; k < kOwned; ++k)
+      mine[k] += (packed >> (8 * k)) & 0xffu;
+  }
+  if (tid == 0) {
+    uint32_t packed = head ? key(idx[0]) : 0u;
+    if ((n - head) & 1)
+      packed += key(idx[n - 1]);
+#pragma unroll
+    for (int k = 0; k < kOwned; ++k)
+      mine[k] += (packed >> (8 * k)) & 0xffu;
+  }
+  // butterfly over the wave, the four counters side by side
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    uint32_t other[kOwned];
+#pragma unroll
+    for (int k = 0; k < kOwned; ++k)
+      other[k] = bpermute(mine[k], lane_id() ^ off);
+#pragma unroll
+    for (int k = 0; k < kOwned; ++k)
+      mine[k] += other[k];
+  }
+  if (tid % kWave == 0)
+#pragma unroll
+    for (int k = 0; k < kOwned; ++k)
+      per_wave[tid / kWave][k] = (int32_t)mine[k];
+  __syncthreads();
+  if (tid < kOwned && base + tid < n_experts) {
+    int32_t sum = 0;
+    for (int w = 0; w < nt / kWave; ++w)
+      sum += per_wave[w][tid];
+    totals[base + tid] = sum;
+  }
+}
+
 // Enqueues histogram and prefix.  any_order: the histogram launch does not wait for
 // the kernel enqueued just before it on the stream (it still starts after everything
 // that kernel waited for); the prefix launch is ordered after both.
@@ -164,4 +237,20 @@ extern "C" int lplb_count_idx(const int64_t *idx, int64_t n_elements,
                "count_idx: idx must be 8-byte aligned");
   return enqueue_count(idx, n_elements, n_experts, n_blocks, counts_by_block,
                        static_cast<hipStream_t>(stream), /*any_order=*/false);
+}
+
+extern "C" int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_experts, int32_t *totals,
+                                 lplb_stream_t stream) {
+  using namespace lplb;
+  LPLB_REQUIRE(n_elements >= 0 && n_experts > 0, LPLB_EINVAL, "count_totals: n_elements=%lld n_experts=%d",
+               (long long)n_elements, n_experts);
+  LPLB_REQUIRE(totals != nullptr && (idx != nullptr || n_elements == 0), LPLB_EINVAL, "count_totals: null pointer");
+  LPLB_REQUIRE((reinterpret_cast<uintptr_t>(idx) & 7) == 0, LPLB_EINVAL, "count_totals: idx must be 8-byte aligned");
+  LPLB_REQUIRE(n_elements <= kTotalsMaxIndices && n_experts <= kTotalsMaxExperts, LPLB_EUNSUPPORTED,
+               "count_totals: serves up to %lld indices and %d experts (use lplb_count_idx beyond)",
+               (long long)kTotalsMaxIndices, kTotalsMaxExperts);
+  launch(expert_totals, dim3((n_experts + kOwned - 1) / kOwned), dim3(1024), 0, static_cast<hipStream_t>(stream), idx,
+         n_elements, n_experts, totals);
+  LPLB_HIP_TRY(hipGetLastError());
+  return LPLB_OK;
 }

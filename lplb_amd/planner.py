@@ -231,13 +231,24 @@ class Planner:
         # With a process group the counts have to be summed over the ranks between histogram and
         # LP (lplb/planner.py:214-216); LP and redirect then run as one plan on the summed counts.
         # (the histogram's table is kept per stream like the plan's other buffers)
-        table = ws.get("group_counts")
-        if table is None or table.device != idx.device:
-            table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32, device=idx.device)
         # (The reference copies the counts before it reduces them, lplb/planner.py:215, because its redirect
-        # reads the same table afterwards.  This table is not read again -- the plan counts its slices
-        # itself -- so the sum may replace its last row.)
-        workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
+        # reads the same table afterwards.  Here nothing reads them again -- the plan counts its slices
+        # itself -- so the sum replaces them, and short batches do without the table per slice altogether.)
+        workload = None
+        if ws.get("group_counts_form") != "table":
+            totals = ws.get("group_totals")
+            if totals is None or totals.device != idx.device:
+                totals = ws["group_totals"] = torch.empty(self.solver.n_experts, dtype=torch.int32, device=idx.device)
+            try:
+                workload = self.solver.count_totals(idx, out=totals)
+            except _native.UnsupportedShape:
+                ws["group_counts_form"] = "table"    # a long batch: histogram and scan
+        if workload is None:
+            table = ws.get("group_counts")
+            if table is None or table.device != idx.device:
+                table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32,
+                                                         device=idx.device)
+            workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
         if not self.deep_ep_initialized:
             torch.distributed.all_reduce(workload, group=self.ep_group)
         out, _o_weight, _by_sm = self.solver.plan(idx, self.r2o, self.o2r, self.phy2log, avail_counter, n_sms,

@@ -58,6 +58,31 @@ def _random_weights(shape: Shape, rng):
     return np.clip(w, 0, 1).astype(np.float32)
 
 
+@pytest.mark.parametrize("n,n_experts,offset", [(65536, 256, 0), (65537, 256, 1), (4099, 30, 0), (1, 7, 0), (0, 64, 0),
+                                                (131072, 1024, 3), (2, 3, 1), (50000, 257, 0)])
+def test_count_totals_matches_oracle(cuda, n, n_experts, offset):
+    """The one-launch totals (what Planner.run feeds the all-reduce with) equal the last row of the table, for
+    masked and out-of-range values, odd lengths, and views that start at an odd multiple of 8 bytes."""
+    rng = np.random.default_rng(n + n_experts)
+    host = rng.integers(-1, n_experts, size=n + offset).astype(np.int64)
+    if n > 10:
+        host[offset + 3] = n_experts          # out of range: not counted
+        host[offset + 7] = -5
+        host[offset + 5:offset + 5 + n // 3] = n_experts - 1      # a hot expert, the last one
+    from lplb_amd._native import CompiledSolver, load
+    lib = load()
+    d_idx = dev(host, cuda)[offset:]
+    totals = torch.full((n_experts,), -9, dtype=torch.int32, device=cuda)
+    rc = lib.lplb_count_totals(d_idx.data_ptr(), n, n_experts, totals.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.lplb_last_error()
+    want = oracle.count_idx(host[offset:], n_experts, 4)[-1]
+    np.testing.assert_array_equal(totals.cpu().numpy(), want)
+    # beyond what it serves it refuses (the caller then runs histogram and scan)
+    some = torch.zeros(2, dtype=torch.int64, device=cuda)
+    assert lib.lplb_count_totals(some.data_ptr(), (1 << 17) + 2, n_experts, totals.data_ptr(), None) == 2
+    assert lib.lplb_count_totals(some.data_ptr(), 2, 1025, totals.data_ptr(), None) == 2
+
+
 @pytest.mark.parametrize("case", ["cube8_ep32", "cube8_ep32_c2", "ring8_ep32", "hypercube16", "torus8x4"])
 @pytest.mark.parametrize("n,n_sms", [(65536, 256), (4099, 7), (300, 256), (1 << 20, 256)])
 def test_map_idx_matches_oracle(cuda, case, n, n_sms):
