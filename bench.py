@@ -149,12 +149,38 @@ def copy_sweep(lib, torch, dev) -> None:
                      "GBs_avg": round(2 * n_bytes / (float(us.mean()) * 1e-6) / 1e9, 1),
                      "frac_of_peak_avg": round(2 * n_bytes / (float(us.mean()) * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
         del src, dst
+    # other shapes of the same copy at the sweep's size (16 MiB each way): what the library's choice rests on
+    n_el, n_pairs, reps = (1 << 24) // 8, 16, 10
+    src = [torch.randint(0, 256, (n_el,), dtype=torch.int64, device=dev) for _ in range(n_pairs)]
+    dst = [torch.empty_like(t) for t in src]
+    n = n_pairs * reps
+    arr = lambda ts: (ctypes.c_void_p * n)(*[ts[i % n_pairs].data_ptr() for i in range(n)])
+    a_src, a_dst = arr(src), arr(dst)
+    shapes = []
+    for loads in (1, 2, 4, 8):
+        for threads in (256, 512, 1024):
+            for barrier, streaming in ((1, 1), (0, 1), (1, 0)):
+                if (barrier, streaming) != (1, 1) and threads != 1024:
+                    continue
+                args = (a_src, a_dst, n_el, n, loads, threads, barrier, streaming)
+                assert lib.lplb_copy_shape_series(*args, None, None, stream) == 0, lib.lplb_last_error()
+                timer = KernelTimer(lib, n)
+                starts, stops = timer.take(n)
+                assert lib.lplb_copy_shape_series(*args, starts, stops, stream) == 0
+                us = timer.times_us(torch)
+                timer.close()
+                shapes.append({"loads_per_lane": loads, "threads": threads, "barrier": bool(barrier),
+                               "streaming": bool(streaming), "workgroups": n_el // (2 * threads * loads),
+                               "avg_us": round(float(us.mean()), 2), "p50_us": round(pct(us, 50), 2),
+                               "min_us": round(float(us.min()), 2)})
+    assert torch.equal(dst[0], src[0])
+    del src, dst
     # time = fixed + bytes / rate, fitted over the sizes from 1 MiB up
     big = [r for r in rows if r["bytes_each_way"] >= 1 << 20]
     x = np.array([2.0 * r["bytes_each_way"] for r in big])
     y = np.array([r["avg_us"] for r in big])
     slope, fixed = np.polyfit(x, y, 1)
-    print(json.dumps({"copy_sweep": rows, "fit_from_1MiB": {"fixed_us": round(float(fixed), 2),
+    print(json.dumps({"copy_sweep": rows, "shapes_at_16MiB": shapes, "fit_from_1MiB": {"fixed_us": round(float(fixed), 2),
                                                            "GBs": round(1e-3 / float(slope), 1)}}))
 
 
@@ -309,25 +335,30 @@ def main() -> None:
     # bytes through a plain copy kernel are the practical ceiling on this box; the two kernels take turns, block
     # of n_buf launches by block, so that whatever drifts during the run treats them alike.
     n_series = n_buf
-    timer = KernelTimer(lib, 2 * reps * n_series)
+    timer = KernelTimer(lib, 3 * reps * n_series)
     ptrs = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
     series_in, series_by, series_out = ptrs(bufs_in), ptrs(tables), ptrs(bufs_out)
     half = n_buf // 2
     copy_in, copy_out = ptrs(bufs_in[half:] + bufs_in[:half]), ptrs(bufs_out[half:] + bufs_out[:half])
-    red_slots, copy_slots = [], []
+    # (a third series: the copy in the redirect's own launch shape, two workgroups of 16 waves per CU and two
+    # 16-byte loads per lane, which is 1 us slower than the copy's best shape)
+    red_slots, copy_slots, twin_slots = [], [], []
     for _ in range(reps):
-        for which, slots in (("redirect", red_slots), ("copy", copy_slots)):
+        for which, slots in (("redirect", red_slots), ("copy", copy_slots), ("twin", twin_slots)):
             starts, stops = timer.take(n_series)
             if which == "redirect":
                 rc = lib.lplb_map_idx_prepared_series(series_in, o_w.data_ptr(), series_by, prepared.data_ptr(), n_idx, 1, G,
                                                       D, C, P, roof_blocks, series_out, n_series, starts, stops, stream)
-            else:
+            elif which == "copy":
                 rc = lib.lplb_copy_calibration_series(copy_in, copy_out, n_idx, n_series, starts, stops, stream)
+            else:
+                rc = lib.lplb_copy_shape_series(copy_in, copy_out, n_idx, n_series, 2, 1024, 1, 1, starts, stops, stream)
             assert rc == 0, lib.lplb_last_error()
             slots.append(timer.used)
     both_us = timer.times_us(torch)
     red_us = np.concatenate([both_us[e - n_series:e] for e in red_slots])
     copy_us = np.concatenate([both_us[e - n_series:e] for e in copy_slots])
+    twin_us = np.concatenate([both_us[e - n_series:e] for e in twin_slots])
     red_avg = float(red_us.mean())
     alg_bytes = n_idx * REDIRECT_BYTES_PER_INDEX
     achieved = alg_bytes / (red_avg * 1e-6) / 1e9
@@ -356,7 +387,9 @@ def main() -> None:
                 "back_to_back_us_per_launch": round(float(np.median(burst)), 2),
                 "copy_kernel_GBs_same_bytes": round(copy_gbs, 1),
                 "copy_kernel_avg_launch_us": round(float(copy_us.mean()), 2),
-                "frac_of_copy_kernel": round(achieved / copy_gbs, 4)}
+                "frac_of_copy_kernel": round(achieved / copy_gbs, 4),
+                "copy_in_the_redirects_launch_shape_avg_us": round(float(twin_us.mean()), 2),
+                "frac_of_copy_in_the_redirects_launch_shape": round(float(twin_us.mean()) / red_avg, 4)}
     extras["redirect_tokens_per_s"] = round(n_idx / (red_avg * 1e-6), 1)
 
     if not args.skip_extras:

@@ -78,6 +78,18 @@ int lplb_copy_calibration_series(const int64_t *const *src, int64_t *const *dst,
                                  int64_t n_elements, int n_launches,
                                  void *const *start_events, void *const *stop_events,
                                  lplb_stream_t stream);
+/*
+ * Measurement aid, no counterpart in the reference: the copy of lplb_copy_calibration in
+ * another shape (loads_per_lane 16-byte loads per lane: 1, 2, 4 or 8; threads per
+ * workgroup: 256, 512 or 1024; with or without a workgroup barrier between loads and
+ * stores; streaming or cached accesses), n_launches times as in the series above.
+ * n_elements must be a multiple of 2 * threads * loads_per_lane.  This is what the choice
+ * of lplb_copy_calibration's own shape rests on (bench.py --copy-sweep prints the table).
+ */
+int lplb_copy_shape_series(const int64_t *const *src, int64_t *const *dst, int64_t n_elements,
+                           int n_launches, int loads_per_lane, int threads, int barrier,
+                           int streaming, void *const *start_events, void *const *stop_events,
+                           lplb_stream_t stream);
 int lplb_map_idx_prepared_series(const int64_t *const *idx, const float *o_weight,
                                  const int32_t *const *counts_by_block, const void *prepared,
                                  int64_t n_elements, int n_group, int group_size,
