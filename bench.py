@@ -438,6 +438,20 @@ def main() -> None:
         h_timer.close()
         extras["histogram_kernel_sweep_us"] = round(hk_us, 2)
         extras["histogram_kernel_sweep_frac_of_peak"] = round(n_idx * HISTOGRAM_BYTES_PER_INDEX / (hk_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+        # the same kernel in a series of its own (every launch timed, no scan behind it): a timed kernel that is
+        # followed at once by another kernel on the stream reads 1.3-1.6 us longer by its own events
+        n_h = 10 * n_buf
+        h_series = KernelTimer(lib, n_h)
+        h_in = (ctypes.c_void_p * n_h)(*[bufs_in[r % n_buf].data_ptr() for r in range(n_h)])
+        h_out = (ctypes.c_void_p * n_h)(*[cu_tables[r % n_buf].data_ptr() for r in range(n_h)])
+        assert lib.lplb_slice_histogram_series(h_in, n_idx, cfg.n_logical, n_sms, h_out, n_h, None, None, stream) == 0
+        starts, stops = h_series.take(n_h)
+        assert lib.lplb_slice_histogram_series(h_in, n_idx, cfg.n_logical, n_sms, h_out, n_h, starts, stops, stream) == 0
+        hs_us = float(h_series.times_us(torch).mean())
+        h_series.close()
+        extras["histogram_kernel_sweep_us_in_a_series_of_its_own"] = round(hs_us, 2)
+        extras["histogram_kernel_sweep_frac_of_peak_in_a_series_of_its_own"] = round(
+            n_idx * HISTOGRAM_BYTES_PER_INDEX / (hs_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
 
         # the whole plan at the sweep shape: histogram of [262144 x 8], LP, redirect (16 B per index)
         sweep_counts_dev = to_dev(sweep.global_counts)

@@ -90,6 +90,16 @@ int lplb_copy_shape_series(const int64_t *const *src, int64_t *const *dst, int64
                            int n_launches, int loads_per_lane, int threads, int barrier,
                            int streaming, void *const *start_events, void *const *stop_events,
                            lplb_stream_t stream);
+/*
+ * Measurement aid, no counterpart in the reference: the first of lplb_count_idx's two kernels
+ * (the histogram per slice, rows not yet summed over the slices) alone, n_launches times as in
+ * the series above.  A kernel that is followed at once by another one on the stream reads
+ * 1.3-1.6 us longer by its own events than in a series of its own; this gives the latter.
+ */
+int lplb_slice_histogram_series(const int64_t *const *idx, int64_t n_elements, int n_experts,
+                                int n_blocks, int32_t *const *counts_by_block, int n_launches,
+                                void *const *start_events, void *const *stop_events,
+                                lplb_stream_t stream);
 int lplb_map_idx_prepared_series(const int64_t *const *idx, const float *o_weight,
                                  const int32_t *const *counts_by_block, const void *prepared,
                                  int64_t n_elements, int n_group, int group_size,

@@ -35,6 +35,7 @@ _SIGNATURES = {
     "lplb_time_next_launch": (None, [_vp, _vp]),
     "lplb_copy_calibration": (_i, [_vp, _vp, _i64, _vp]),
     "lplb_copy_calibration_series": (_i, [_vp, _vp, _i64, _i, _vp, _vp, _vp]),
+    "lplb_slice_histogram_series": (_i, [_vp, _i64, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "lplb_copy_shape_series": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_map_idx_prepared_series": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),

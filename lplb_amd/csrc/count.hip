@@ -254,3 +254,29 @@ extern "C" int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_e
   LPLB_HIP_TRY(hipGetLastError());
   return LPLB_OK;
 }
+
+// Measurement aid: the histogram kernel alone (no scan behind it), n_launches times, launch r on idx[r] and
+// counts_by_block[r], each recording its own begin and end into start_events[r] / stop_events[r].
+extern "C" int lplb_slice_histogram_series(const int64_t *const *idx, int64_t n_elements, int n_experts, int n_blocks,
+                                           int32_t *const *counts_by_block, int n_launches, void *const *start_events,
+                                           void *const *stop_events, lplb_stream_t stream) {
+  using namespace lplb;
+  LPLB_REQUIRE(idx && counts_by_block && n_launches >= 0, LPLB_EINVAL, "slice_histogram_series: null pointer or negative count");
+  LPLB_REQUIRE(n_elements > 0 && n_elements <= INT32_MAX && n_experts > 0 && n_blocks > 0 &&
+                   sizeof(int32_t) * (size_t)n_experts <= 64 * 1024,
+               LPLB_EINVAL, "slice_histogram_series: n_elements=%lld n_experts=%d n_blocks=%d", (long long)n_elements,
+               n_experts, n_blocks);
+  const size_t lds = sizeof(int32_t) * (size_t)n_experts;
+  const int64_t per = slice_len(n_elements, n_blocks);
+  const int64_t batches = (per / 2 + kLoadsInFlight - 1) / kLoadsInFlight;
+  const int threads = batches <= 256 ? 256 : batches <= 512 ? 512 : 1024;
+  for (int r = 0; r < n_launches; ++r) {
+    LPLB_REQUIRE(idx[r] && counts_by_block[r] && (reinterpret_cast<uintptr_t>(idx[r]) & 7) == 0, LPLB_EINVAL,
+                 "slice_histogram_series: bad pointer in launch %d", r);
+    lplb_time_next_launch(start_events ? start_events[r] : nullptr, stop_events ? stop_events[r] : nullptr);
+    launch(slice_histogram, dim3(n_blocks), dim3(threads), lds, static_cast<hipStream_t>(stream), idx[r], n_elements,
+           n_experts, per, counts_by_block[r]);
+    LPLB_HIP_TRY(hipGetLastError());
+  }
+  return LPLB_OK;
+}

@@ -1370,6 +1370,18 @@ def test_series_aids_equal_single_calls(cuda):
     torch.cuda.synchronize()
     for o, w in zip(back, idx):
         assert torch.equal(o, w)
+    # the copy in another launch shape, and the histogram kernel without the scan behind it
+    back = [torch.zeros_like(t) for t in idx]
+    assert lib.lplb_copy_shape_series(ptrs(idx), ptrs(back), n, 3, 4, 256, 1, 0, None, None, None) == 0
+    rows = [torch.full_like(b, -3) for b in by]
+    assert lib.lplb_slice_histogram_series(ptrs(idx), n, shape.n_logical, n_sms, ptrs(rows), 3, None, None, None) == 0
+    torch.cuda.synchronize()
+    for o, w in zip(back, idx):
+        assert torch.equal(o, w)
+    for r, b in zip(rows, by):
+        assert torch.equal(torch.cumsum(r, dim=0, dtype=torch.int32), b)
+    assert lib.lplb_copy_shape_series(ptrs(idx), ptrs(back), n, 3, 3, 256, 1, 0, None, None, None) == 1   # loads: 1, 2, 4 or 8
+    assert lib.lplb_copy_shape_series(ptrs(idx), ptrs(back), n + 2, 3, 4, 256, 1, 0, None, None, None) == 1   # whole tiles only
 
 
 def test_kernel_timestamp_hook(cuda):
