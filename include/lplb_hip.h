@@ -130,11 +130,14 @@ int lplb_count_idx(const int64_t *idx, int64_t n_elements, int n_experts,
  * Planner.run with a process group, which needs the counts for the all-reduce
  * ahead of the plan and no table (lplb/planner.py:209-216 gets them from count_idx).
  * Every workgroup reads the whole batch, so this is for short batches:
- * n_elements <= 131072 and n_experts <= 1024, LPLB_EUNSUPPORTED beyond (callers
- * then use lplb_count_idx).
+ * n_elements <= LPLB_COUNT_TOTALS_MAX_INDICES and n_experts <=
+ * LPLB_COUNT_TOTALS_MAX_EXPERTS, LPLB_EUNSUPPORTED beyond (callers then use
+ * lplb_count_idx).
  *
  *   totals           int32 [n_experts], out
  */
+#define LPLB_COUNT_TOTALS_MAX_INDICES 131072
+#define LPLB_COUNT_TOTALS_MAX_EXPERTS 1024
 int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_experts,
                       int32_t *totals, lplb_stream_t stream);
 

@@ -18,6 +18,9 @@ import torch
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
 ABI_VERSION = 6
+# limits of lplb_count_totals (LPLB_COUNT_TOTALS_MAX_* of include/lplb_hip.h)
+COUNT_TOTALS_MAX_INDICES = 131072
+COUNT_TOTALS_MAX_EXPERTS = 1024
 
 STEP_REFERENCE_WINDOW = 0
 STEP_FULL_MAX = 1

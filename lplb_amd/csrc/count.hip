@@ -133,8 +133,8 @@ __global__ __launch_bounds__(kScanBands *kScanCols) void prefix_over_slices(
 // long as the launch itself, against two launches for histogram and scan.  A lane keeps four counters;
 // the values of a batch of loads are first added up in one register, a byte per owned expert.
 constexpr int kOwned = 4;
-constexpr int64_t kTotalsMaxIndices = 1 << 17;   // per call; beyond, the two-kernel form is faster
-constexpr int kTotalsMaxExperts = 1024;
+constexpr int64_t kTotalsMaxIndices = LPLB_COUNT_TOTALS_MAX_INDICES;   // per call; beyond, the two-kernel form is faster
+constexpr int kTotalsMaxExperts = LPLB_COUNT_TOTALS_MAX_EXPERTS;
 
 __global__ __launch_bounds__(1024) void expert_totals(const int64_t *__restrict__ idx, int64_t n, int n_experts,
                                                       int32_t *__restrict__ totals) {

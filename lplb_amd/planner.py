@@ -234,16 +234,12 @@ class Planner:
         # (The reference copies the counts before it reduces them, lplb/planner.py:215, because its redirect
         # reads the same table afterwards.  Here nothing reads them again -- the plan counts its slices
         # itself -- so the sum replaces them, and short batches do without the table per slice altogether.)
-        workload = None
-        if ws.get("group_counts_form") != "table":
+        if idx.numel() <= _native.COUNT_TOTALS_MAX_INDICES and self.solver.n_experts <= _native.COUNT_TOTALS_MAX_EXPERTS:
             totals = ws.get("group_totals")
             if totals is None or totals.device != idx.device:
                 totals = ws["group_totals"] = torch.empty(self.solver.n_experts, dtype=torch.int32, device=idx.device)
-            try:
-                workload = self.solver.count_totals(idx, out=totals)
-            except _native.UnsupportedShape:
-                ws["group_counts_form"] = "table"    # a long batch: histogram and scan
-        if workload is None:
+            workload = self.solver.count_totals(idx, out=totals)
+        else:                                        # a long batch: histogram and scan
             table = ws.get("group_counts")
             if table is None or table.device != idx.device:
                 table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32,

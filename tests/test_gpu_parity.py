@@ -1036,6 +1036,18 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
     lw, by_sm = planner.count_workload(t["idx"], 256)
     o_weight, _ = planner.solve_probs(lw, avail2)
     assert torch.equal(planner.weighted_select_target(t["idx"], o_weight, by_sm, 256), out)
+    # a batch too long for the one-launch totals takes histogram + scan, then a short one again
+    from lplb_amd import _native
+    long_idx = t["idx"].repeat(3, 1)
+    assert t["idx"].numel() <= _native.COUNT_TOTALS_MAX_INDICES < long_idx.numel()
+    for batch, times in ((long_idx, 3), (t["idx"], 1)):
+        avail.zero_(), avail2.zero_()
+        got = planner.run(batch, avail, 256)
+        want, _, _ = solver.plan(batch, t["r2o"], t["o2r"], t["phy2log"], avail2, 256,
+                                 global_counts=times * dev(local, cuda) + others)
+        assert int(avail[0]) == int(avail2[0]) == shape.n_group, (times, int(avail[0]), int(avail2[0]))
+        assert torch.equal(got, want), (times, int((got != want).sum()))
+    assert len(calls) == 4   # run, solve_probs, and the two runs above
 
 
 @pytest.mark.parametrize("use_global", [True, False])

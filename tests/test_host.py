@@ -226,6 +226,8 @@ def test_library_exports_every_declared_symbol():
     assert lib.lplb_abi_version() == _native.ABI_VERSION == 6
     header = (ROOT / "include" / "lplb_hip.h").read_text()
     assert f"#define LPLB_ABI_VERSION {_native.ABI_VERSION}" in header
+    assert f"#define LPLB_COUNT_TOTALS_MAX_INDICES {_native.COUNT_TOTALS_MAX_INDICES}\n" in header
+    assert f"#define LPLB_COUNT_TOTALS_MAX_EXPERTS {_native.COUNT_TOTALS_MAX_EXPERTS}\n" in header
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
