@@ -384,6 +384,9 @@ def main() -> None:
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_us": round(red_avg, 2),
                 "p50_launch_us": round(pct(red_us, 50), 2), "p99_launch_us": round(pct(red_us, 99), 2),
                 "launches_timed": int(red_us.size), "distinct_buffer_pairs": n_buf,
+                # launches that read 2 us or more above the median: what separates avg from p50 (the copy has them too)
+                "launches_2us_above_p50_frac": round(float(np.mean(red_us > pct(red_us, 50) + 2.0)), 4),
+                "copy_launches_2us_above_p50_frac": round(float(np.mean(copy_us > pct(copy_us, 50) + 2.0)), 4),
                 "back_to_back_us_per_launch": round(float(np.median(burst)), 2),
                 "copy_kernel_GBs_same_bytes": round(copy_gbs, 1),
                 "copy_kernel_avg_launch_us": round(float(copy_us.mean()), 2),
