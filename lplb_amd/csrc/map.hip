@@ -743,10 +743,6 @@ __global__ __launch_bounds__(kMaxWaves *kWave, KP >= 4 ? 4 : 8) void redirect_pa
   LPLB_MAP_STAMP(10);
 }
 
-#ifdef LPLB_TUNING
-// Tuning builds only: force the launch shape of the redirect (0 = choose as usual).
-int g_force_waves = 0, g_force_k = 0, g_force_pairs = 0;   // pairs: 1 = always where possible, -1 = never
-#endif
 
 template <int K, bool WRAP, bool TAIL, bool SINGLE>
 static hipError_t launch_redirect_variant(const MapArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t s) {
@@ -870,20 +866,10 @@ static int map_checked(const int64_t *idx, const float *o_weight, const int32_t 
     bool pairs = prepared != nullptr && !wrap && runs <= (int64_t)kMaxWaves * kMaxPairRuns && a.n_rep <= kPairMaxSets &&
                  n_elements <= kPairMaxTotal && a.n_ranks * a.P <= kPairMaxSlots &&
                  ((reinterpret_cast<uintptr_t>(idx) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-    // as many waves as the slice has runs, up to 16 (two such workgroups fill a CU's wave slots: a copy
-    // is fastest in that shape too), then 2 and 4 runs per wave
+    // as many waves as the slice has runs, up to 16 (two such workgroups fill a CU's wave slots, and one's
+    // ranking overlaps the other's loads and stores), then 2 and 4 runs per wave
     int kp = runs > 2 * kMaxWaves ? 4 : runs > kMaxWaves ? 2 : 1;
     int n_waves = (int)((runs + kp - 1) / kp);
-#ifdef LPLB_TUNING
-    if (g_force_pairs < 0)
-      pairs = false;
-    if (g_force_pairs > 0 && g_force_k > 0)
-      kp = g_force_k;
-    if (g_force_pairs > 0 && g_force_waves > 0)
-      n_waves = g_force_waves;
-    else
-      n_waves = (int)((runs + kp - 1) / kp);
-#endif
     if (pairs && n_waves <= kMaxWaves && (int64_t)n_waves * kp >= runs &&
         pairs_lds_bytes(a.n_logical, a.n_rep, n_waves, kp) <= kLdsLimit) {
       LPLB_HIP_TRY(launch_pairs(a, n_waves, kp, pairs_lds_bytes(a.n_logical, a.n_rep, n_waves, kp), s));
@@ -903,12 +889,6 @@ static int map_checked(const int64_t *idx, const float *o_weight, const int32_t 
   int n_waves = chunks < max_waves ? (int)chunks : max_waves;
   const int64_t per_wave = (chunks + n_waves - 1) / n_waves;
   int k = per_wave >= 8 ? 4 : per_wave >= 3 ? 2 : 1;
-#ifdef LPLB_TUNING
-  if (g_force_waves > 0)
-    n_waves = min(g_force_waves, kMaxWaves);
-  if (g_force_k > 0)
-    k = g_force_k;
-#endif
   while (k > 1 && map_lds_bytes(a.n_logical, a.n_rep, n_waves, k) > kLdsLimit)
     k >>= 1;
   while (n_waves > 1 && map_lds_bytes(a.n_logical, a.n_rep, n_waves, k) > kLdsLimit)
@@ -936,13 +916,6 @@ static int map_checked(const int64_t *idx, const float *o_weight, const int32_t 
 
 } // namespace lplb
 
-#ifdef LPLB_TUNING
-extern "C" void lplb_debug_force_redirect_shape(int waves, int k) {
-  lplb::g_force_waves = waves;
-  lplb::g_force_k = k;
-}
-extern "C" void lplb_debug_force_redirect_pairs(int mode) { lplb::g_force_pairs = mode; }
-#endif
 
 extern "C" int lplb_map_idx(const int64_t *idx, const float *o_weight,
                             const int32_t *counts_by_block, const int32_t *o2r,

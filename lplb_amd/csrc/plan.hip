@@ -830,14 +830,6 @@ static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *don
   static KernelFootprint footprint;
   const int fit = workgroups_per_cu(reinterpret_cast<const void *>(kernel), footprint, WAVES, lds);
   const int n_workgroups = a.n_slices + a.n_lp_workgroups;
-#ifdef LPLB_TUNING
-  {
-    hipFuncAttributes attr;
-    (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel));
-    fprintf(stderr, "plan variant <%d,%d,%d,K=%d,W=%d>: %d workgroups, lds %zu, %d fit a CU, %d CUs (numRegs %d, static LDS %zu)\n",
-            GM, DM, (int)EXACT, K, WAVES, n_workgroups, lds, fit, d->n_cus, attr.numRegs, attr.sharedSizeBytes);
-  }
-#endif
   if (fit <= 0 || n_workgroups > (int)(kResidencyBudget * fit * d->n_cus))
     return LPLB_OK;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -847,9 +839,6 @@ static int launch_plan_variant(PlanArgs &a, size_t lds, hipStream_t s, bool *don
   const float cost = (float)n_workgroups / (float)(fit * d->n_cus);
   std::lock_guard<std::mutex> lock(g_plan_guard);   // held over the launch: admission and launch order agree
   const int slot = admit_launch(*d, s, cost, capturing);
-#ifdef LPLB_TUNING
-  fprintf(stderr, "  admission: slot %d, cost %.3f\n", slot, cost);
-#endif
   if (slot < 0)
     return LPLB_OK;
   PlanSlot &ps = d->slots[slot];
