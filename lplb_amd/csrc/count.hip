@@ -19,9 +19,14 @@ constexpr int kLoadsInFlight = 4;   // 16-byte loads a thread issues before it c
 
 // COPIES histograms side by side, lane l counts into copy l % COPIES: lanes of one instruction that
 // hold the same expert are served one after the other by the LDS, and at Zipf(1.0) the hottest expert
-// has ten of a wave's 64 tokens.  (Measured at [262144 x 8] in 256 slices, kernel alone: one copy
-// 5.3 us, two 5.1, four 4.9, eight 4.8; a copy per wave instead of per lane: no gain.)
+// has ten of a wave's 64 tokens.  The copies start 4 banks apart (a stride of 4 modulo the 32 banks),
+// so that the counters of one expert sit in eight different banks.  (Measured at [262144 x 8] in 256
+// slices, kernel alone: one copy 5.3 us, two 5.1, four 4.9, eight 4.8, eight in different banks 4.6;
+// a copy per wave instead of per lane: no gain.)
 constexpr int kHistogramCopies = 8;
+__host__ __device__ constexpr int histogram_stride(int n_experts, int copies) {
+  return copies > 1 ? ((n_experts + 31) & ~31) + 4 : n_experts;
+}
 
 template <int COPIES>
 __global__ __launch_bounds__(1024) void slice_histogram(
@@ -31,7 +36,8 @@ __global__ __launch_bounds__(1024) void slice_histogram(
   fetch_arguments_now(idx, n, n_experts, per, counts);
   const int tid = threadIdx.x, nt = blockDim.x;
   const int p = blockIdx.x;
-  int32_t *mine = hist + (tid % COPIES) * n_experts;
+  const int stride = histogram_stride(n_experts, COPIES);
+  int32_t *mine = hist + (tid % COPIES) * stride;
   auto count = [&](int64_t v) {
     if ((uint64_t)v < (uint64_t)n_experts)
       atomicAdd(&mine[(int)v], 1);
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(1024) void slice_histogram(
     const int64_t i = tid + (int64_t)u * nt;
     first[u] = i < n_pairs ? __builtin_nontemporal_load(pairs + i) : i64x2{-1, -1};
   }
-  for (int e = tid; e < COPIES * n_experts; e += nt)
+  for (int e = tid; e < COPIES * stride; e += nt)
     hist[e] = 0;
   __syncthreads();
 #pragma unroll
@@ -84,12 +90,13 @@ __global__ __launch_bounds__(1024) void slice_histogram(
     int32_t sum = 0;
 #pragma unroll
     for (int k = 0; k < COPIES; ++k)
-      sum += hist[k * n_experts + e];
+      sum += hist[k * stride + e];
     row[e] = sum;
   }
 }
 
-// The launch both callers share: eight copies while they fit the 64 KiB of LDS a kernel gets unasked, else one.
+// The launch both callers share: eight copies while they fit the 64 KiB of LDS a kernel gets unasked
+// (up to 2016 experts), else one.
 static int launch_slice_histogram(const int64_t *idx, int64_t n_elements, int n_experts, int n_blocks, int32_t *counts,
                                   hipStream_t s, unsigned flags) {
   const size_t one = sizeof(int32_t) * (size_t)n_experts;
@@ -99,9 +106,10 @@ static int launch_slice_histogram(const int64_t *idx, int64_t n_elements, int n_
   // way, so a slice gets as many threads as cover it in one such batch, up to 1024
   const int64_t batches = (per / 2 + kLoadsInFlight - 1) / kLoadsInFlight;
   const int threads = batches <= 256 ? 256 : batches <= 512 ? 512 : 1024;
-  if (one * kHistogramCopies <= 64 * 1024)
-    launch_with_flags(slice_histogram<kHistogramCopies>, dim3(n_blocks), dim3(threads), one * kHistogramCopies, s, flags,
-                      idx, n_elements, n_experts, per, counts);
+  const size_t copies = sizeof(int32_t) * (size_t)kHistogramCopies * histogram_stride(n_experts, kHistogramCopies);
+  if (copies <= 64 * 1024)
+    launch_with_flags(slice_histogram<kHistogramCopies>, dim3(n_blocks), dim3(threads), copies, s, flags, idx,
+                      n_elements, n_experts, per, counts);
   else
     launch_with_flags(slice_histogram<1>, dim3(n_blocks), dim3(threads), one, s, flags, idx, n_elements, n_experts, per,
                       counts);

@@ -34,8 +34,8 @@ def solver_for(s: Shape) -> CompiledSolver:
 @pytest.mark.parametrize("n,n_experts,n_sms", [
     (4096 * 8, 256, 256), (65536, 256, 100), (0, 256, 8), (1, 32, 4), (255, 32, 3), (257, 32, 3),
     (1000003, 256, 256), (70001, 1000, 37), (65536, 256, 1), (8192 * 8, 256, 304),
-    # the LDS histogram is kept in eight copies up to 2048 experts and in one beyond
-    (300007, 2048, 64), (300007, 2049, 64), (100003, 5000, 19), (40000, 16384, 5),
+    # the LDS histogram is kept in eight copies up to 2016 experts and in one beyond
+    (300007, 2016, 64), (300007, 2017, 64), (100003, 5000, 19), (40000, 16384, 5), (99991, 33, 7), (99991, 1000, 256),
 ])
 def test_count_idx_matches_oracle(cuda, n, n_experts, n_sms):
     rng = np.random.default_rng(n + n_experts + n_sms)
