@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define LPLB_ABI_VERSION 6
+#define LPLB_ABI_VERSION 7
 
 #define LPLB_OK 0
 #define LPLB_EINVAL 1      /* bad argument (null pointer, negative size, ...) */
@@ -140,6 +140,25 @@ int lplb_count_idx(const int64_t *idx, int64_t n_elements, int n_experts,
 #define LPLB_COUNT_TOTALS_MAX_EXPERTS 1024
 int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_experts,
                       int32_t *totals, lplb_stream_t stream);
+
+/*
+ * The same counts, ADDED to what `totals` holds, in one kernel launch of a few
+ * workgroups: slices of 8192 indices count into LDS and add what they found with
+ * device-wide atomic adds (n_elements <= LPLB_COUNT_TOTALS_MAX_INDICES: every
+ * slice updates every counter, and updates of one line of memory queue up).
+ * No counterpart in the reference.  The caller hands
+ * in a vector that is zero (or holds counts to add to); so that it never has
+ * to zero one itself, the launch also sets `clear` to zero if that is given:
+ * a caller keeps two vectors and swaps them from call to call (Planner.run with
+ * a process group does; a call that is captured into a graph must not rely on
+ * that, since a replay starts with the vectors as the last replay left them).
+ * n_experts * 4 bytes must fit 64 KiB of LDS (LPLB_EUNSUPPORTED beyond).
+ *
+ *   totals           int32 [n_experts], in/out, 8-byte aligned
+ *   clear            int32 [n_experts], out (all zero), or NULL; not `totals`
+ */
+int lplb_count_totals_add(const int64_t *idx, int64_t n_elements, int n_experts,
+                          int32_t *totals, int32_t *clear, lplb_stream_t stream);
 
 /*
  * Builds and solves one LP per EP group: minimise the maximum per-rank load by

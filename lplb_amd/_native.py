@@ -17,7 +17,7 @@ import torch
 
 _PKG = Path(__file__).resolve().parent
 LIB_PATH = _PKG / "liblplb_hip.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 # limits of lplb_count_totals (LPLB_COUNT_TOTALS_MAX_* of include/lplb_hip.h)
 COUNT_TOTALS_MAX_INDICES = 131072
 COUNT_TOTALS_MAX_EXPERTS = 1024
@@ -43,6 +43,7 @@ _SIGNATURES = {
     "lplb_map_idx_prepared_series": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "lplb_count_idx": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
     "lplb_count_totals": (_i, [_vp, _i64, _i, _vp, _vp]),
+    "lplb_count_totals_add": (_i, [_vp, _i64, _i, _vp, _vp, _vp]),
     "lplb_solve": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_solve_batched": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "lplb_map_idx": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
@@ -278,6 +279,20 @@ class CompiledSolver:
                      "out: int32 [n_experts], contiguous, on the GPU")
         _check(self.lib.lplb_count_totals(idx.data_ptr(), idx.numel(), self.n_experts, out.data_ptr(), _stream(idx)))
         return out
+
+    def count_totals_add(self, idx: torch.Tensor, totals: torch.Tensor, clear: torch.Tensor | None = None) -> torch.Tensor:
+        """Adds this GPU's tokens per logical expert to ``totals`` (which the caller has zeroed), one kernel launch
+        of a few workgroups (short batches only: UnsupportedShape beyond 131072 indices); the same launch sets
+        ``clear`` to zero, so a caller that swaps two vectors from call to call never zeroes one itself.  No
+        counterpart in the reference."""
+        _require(idx.dtype == torch.int64 and idx.is_cuda and idx.is_contiguous(), "idx is a contiguous int64 GPU tensor")
+        for name, t in (("totals", totals), ("clear", clear)):
+            _require(t is None or (t.dtype == torch.int32 and t.is_cuda and t.is_contiguous() and
+                                   t.numel() == self.n_experts and t.device == idx.device),
+                     f"{name}: int32 [n_experts], contiguous, on idx's GPU")
+        _check(self.lib.lplb_count_totals_add(idx.data_ptr(), idx.numel(), self.n_experts, totals.data_ptr(),
+                                              None if clear is None else clear.data_ptr(), _stream(idx)))
+        return totals
 
     # -- csrc/plugin.cpp:602-660 -------------------------------------------------
     def map_idx(self, mapping_idx: torch.Tensor, o_weight: torch.Tensor, local_workload_split_by_sm: torch.Tensor,

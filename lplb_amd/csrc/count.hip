@@ -28,12 +28,15 @@ __host__ __device__ constexpr int histogram_stride(int n_experts, int copies) {
   return copies > 1 ? ((n_experts + 31) & ~31) + 4 : n_experts;
 }
 
-template <int COPIES>
+// TOTALS: instead of writing its row, a slice adds its counts to the one vector `counts` [n_experts]
+// (device-wide atomic adds, none for an expert the slice has no token of), and the launch sets the
+// vector `clear` (if given) to zero -- a caller that takes two vectors in turn never has to zero one.
+template <int COPIES, bool TOTALS>
 __global__ __launch_bounds__(1024) void slice_histogram(
     const int64_t *__restrict__ idx, int64_t n, int n_experts, int64_t per,
-    int32_t *__restrict__ counts) {
+    int32_t *__restrict__ counts, int32_t *__restrict__ clear) {
   extern __shared__ int32_t hist[];
-  fetch_arguments_now(idx, n, n_experts, per, counts);
+  fetch_arguments_now(idx, n, n_experts, per, counts, clear);
   const int tid = threadIdx.x, nt = blockDim.x;
   const int p = blockIdx.x;
   const int stride = histogram_stride(n_experts, COPIES);
@@ -61,6 +64,10 @@ __global__ __launch_bounds__(1024) void slice_histogram(
   }
   for (int e = tid; e < COPIES * stride; e += nt)
     hist[e] = 0;
+  if constexpr (TOTALS)
+    if (clear)
+      for (int64_t e = (int64_t)p * nt + tid; e < n_experts; e += (int64_t)gridDim.x * nt)
+        clear[e] = 0;
   __syncthreads();
 #pragma unroll
   for (int u = 0; u < kLoadsInFlight; ++u) {
@@ -85,22 +92,45 @@ __global__ __launch_bounds__(1024) void slice_histogram(
   if (tid == 0 && ((end - begin - head) & 1))
     count(idx[end - 1]);
   __syncthreads();
-  int32_t *row = counts + (int64_t)p * n_experts;
+  int32_t *row = TOTALS ? counts : counts + (int64_t)p * n_experts;
   for (int e = tid; e < n_experts; e += nt) {
     int32_t sum = 0;
 #pragma unroll
     for (int k = 0; k < COPIES; ++k)
       sum += hist[k * stride + e];
-    row[e] = sum;
+    if constexpr (!TOTALS)
+      row[e] = sum;
+  }
+  if constexpr (TOTALS) {
+    // Two counters per atomic add: updates of one 64-byte line of memory are served one after the other
+    // (about 14 ns each), and every slice updates every line, so the number of updates is what this
+    // costs.  A counter stays below 2^31, so the low half never carries into the high one.
+    unsigned long long *both = reinterpret_cast<unsigned long long *>(row);
+    for (int e2 = tid; 2 * e2 < n_experts; e2 += nt) {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int k = 0; k < COPIES; ++k) {
+        lo += (uint32_t)hist[k * stride + 2 * e2];
+        hi += 2 * e2 + 1 < n_experts ? (uint32_t)hist[k * stride + 2 * e2 + 1] : 0u;
+      }
+      if (2 * e2 + 1 < n_experts) {
+        if ((lo | hi) != 0)
+          __hip_atomic_fetch_add(both + e2, ((unsigned long long)hi << 32) | lo, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+      } else if (lo != 0) {
+        __hip_atomic_fetch_add(row + 2 * e2, (int32_t)lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
   }
 }
 
-// The launch both callers share: eight copies while they fit the 64 KiB of LDS a kernel gets unasked
-// (up to 2016 experts), else one.
+// The launch all callers share: eight copies while they fit the 64 KiB of LDS a kernel gets unasked
+// (up to 2016 experts), else one.  TOTALS as in the kernel.
+template <bool TOTALS>
 static int launch_slice_histogram(const int64_t *idx, int64_t n_elements, int n_experts, int n_blocks, int32_t *counts,
-                                  hipStream_t s, unsigned flags) {
+                                  int32_t *clear, hipStream_t s, unsigned flags) {
   const size_t one = sizeof(int32_t) * (size_t)n_experts;
-  LPLB_REQUIRE(one <= 64 * 1024, LPLB_EUNSUPPORTED, "count_idx: n_experts=%d does not fit the LDS histogram", n_experts);
+  LPLB_REQUIRE(one <= 64 * 1024, LPLB_EUNSUPPORTED, "n_experts=%d does not fit the LDS histogram", n_experts);
   const int64_t per = slice_len(n_elements, n_blocks);
   // one 16-byte load per thread covers 2 indices; a thread has kLoadsInFlight of them under
   // way, so a slice gets as many threads as cover it in one such batch, up to 1024
@@ -108,11 +138,11 @@ static int launch_slice_histogram(const int64_t *idx, int64_t n_elements, int n_
   const int threads = batches <= 256 ? 256 : batches <= 512 ? 512 : 1024;
   const size_t copies = sizeof(int32_t) * (size_t)kHistogramCopies * histogram_stride(n_experts, kHistogramCopies);
   if (copies <= 64 * 1024)
-    launch_with_flags(slice_histogram<kHistogramCopies>, dim3(n_blocks), dim3(threads), copies, s, flags, idx,
-                      n_elements, n_experts, per, counts);
+    launch_with_flags(slice_histogram<kHistogramCopies, TOTALS>, dim3(n_blocks), dim3(threads), copies, s, flags, idx,
+                      n_elements, n_experts, per, counts, clear);
   else
-    launch_with_flags(slice_histogram<1>, dim3(n_blocks), dim3(threads), one, s, flags, idx, n_elements, n_experts, per,
-                      counts);
+    launch_with_flags(slice_histogram<1, TOTALS>, dim3(n_blocks), dim3(threads), one, s, flags, idx, n_elements,
+                      n_experts, per, counts, clear);
   LPLB_HIP_TRY(hipGetLastError());
   return LPLB_OK;
 }
@@ -245,8 +275,8 @@ __global__ __launch_bounds__(1024) void expert_totals(const int64_t *__restrict_
 // that kernel waited for); the prefix launch is ordered after both.
 int enqueue_count(const int64_t *idx, int64_t n_elements, int n_experts, int n_blocks,
                   int32_t *counts_by_block, hipStream_t s, bool any_order) {
-  const int rc = launch_slice_histogram(idx, n_elements, n_experts, n_blocks, counts_by_block, s,
-                                        any_order ? hipExtAnyOrderLaunch : 0u);
+  const int rc = launch_slice_histogram<false>(idx, n_elements, n_experts, n_blocks, counts_by_block, nullptr, s,
+                                               any_order ? hipExtAnyOrderLaunch : 0u);
   if (rc != LPLB_OK)
     return rc;
   launch(prefix_over_slices, dim3((n_experts + kScanCols - 1) / kScanCols), dim3(kScanBands * kScanCols), 0, s,
@@ -289,6 +319,25 @@ extern "C" int lplb_count_totals(const int64_t *idx, int64_t n_elements, int n_e
   return LPLB_OK;
 }
 
+extern "C" int lplb_count_totals_add(const int64_t *idx, int64_t n_elements, int n_experts, int32_t *totals,
+                                     int32_t *clear, lplb_stream_t stream) {
+  using namespace lplb;
+  LPLB_REQUIRE(n_elements >= 0 && n_elements <= INT32_MAX && n_experts > 0, LPLB_EINVAL,
+               "count_totals_add: n_elements=%lld n_experts=%d", (long long)n_elements, n_experts);
+  LPLB_REQUIRE(totals != nullptr && (idx != nullptr || n_elements == 0), LPLB_EINVAL, "count_totals_add: null pointer");
+  LPLB_REQUIRE(totals != clear, LPLB_EINVAL, "count_totals_add: totals and clear are the same vector");
+  LPLB_REQUIRE(((reinterpret_cast<uintptr_t>(idx) | reinterpret_cast<uintptr_t>(totals)) & 7) == 0, LPLB_EINVAL,
+               "count_totals_add: idx and totals must be 8-byte aligned");
+  LPLB_REQUIRE(n_elements <= kTotalsMaxIndices, LPLB_EUNSUPPORTED,
+               "count_totals_add: serves up to %lld indices (use lplb_count_idx beyond)", (long long)kTotalsMaxIndices);
+  // Slices of 8192 indices (1024 threads with four 16-byte loads each): at most 16 of them, because every
+  // slice updates every line of the totals and those updates queue up.
+  const int64_t wanted = (n_elements + 8191) / 8192;
+  const int n_blocks = (int)(wanted < 1 ? 1 : wanted);
+  return launch_slice_histogram<true>(idx, n_elements, n_experts, n_blocks, totals, clear,
+                                      static_cast<hipStream_t>(stream), 0u);
+}
+
 // Measurement aid: the histogram kernel alone (no scan behind it), n_launches times, launch r on idx[r] and
 // counts_by_block[r], each recording its own begin and end into start_events[r] / stop_events[r].
 extern "C" int lplb_slice_histogram_series(const int64_t *const *idx, int64_t n_elements, int n_experts, int n_blocks,
@@ -304,8 +353,8 @@ extern "C" int lplb_slice_histogram_series(const int64_t *const *idx, int64_t n_
     LPLB_REQUIRE(idx[r] && counts_by_block[r] && (reinterpret_cast<uintptr_t>(idx[r]) & 7) == 0, LPLB_EINVAL,
                  "slice_histogram_series: bad pointer in launch %d", r);
     lplb_time_next_launch(start_events ? start_events[r] : nullptr, stop_events ? stop_events[r] : nullptr);
-    const int rc = launch_slice_histogram(idx[r], n_elements, n_experts, n_blocks, counts_by_block[r],
-                                          static_cast<hipStream_t>(stream), 0u);
+    const int rc = launch_slice_histogram<false>(idx[r], n_elements, n_experts, n_blocks, counts_by_block[r], nullptr,
+                                                 static_cast<hipStream_t>(stream), 0u);
     if (rc != LPLB_OK) {
       lplb_time_next_launch(nullptr, nullptr);
       return rc;

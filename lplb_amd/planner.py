@@ -233,17 +233,30 @@ class Planner:
         # (the histogram's table is kept per stream like the plan's other buffers)
         # (The reference copies the counts before it reduces them, lplb/planner.py:215, because its redirect
         # reads the same table afterwards.  Here nothing reads them again -- the plan counts its slices
-        # itself -- so the sum replaces them, and short batches do without the table per slice altogether.)
-        if idx.numel() <= _native.COUNT_TOTALS_MAX_INDICES and self.solver.n_experts <= _native.COUNT_TOTALS_MAX_EXPERTS:
+        # itself -- so the sum replaces them, and no table per slice is made at all.)
+        n_experts = self.solver.n_experts
+        short = idx.numel() <= _native.COUNT_TOTALS_MAX_INDICES
+        if not capturing and short and n_experts * 4 <= 64 * 1024:
+            # one launch adds the batch's counts to a zeroed vector and zeroes the vector of the call before
+            pair = ws.get("group_totals_pair")
+            if pair is None or pair[0].device != idx.device:
+                pair = ws["group_totals_pair"] = [torch.zeros(n_experts, dtype=torch.int32, device=idx.device)
+                                                  for _ in range(2)]
+                ws["group_totals_turn"] = 0
+            turn = ws["group_totals_turn"]
+            workload = self.solver.count_totals_add(idx, pair[turn], clear=pair[1 - turn])
+            ws["group_totals_turn"] = 1 - turn
+        elif short and n_experts <= _native.COUNT_TOTALS_MAX_EXPERTS:
+            # (a captured call replays with the vectors as the last replay left them: it takes the launch in
+            # which every workgroup owns four experts and nothing has to be zero beforehand)
             totals = ws.get("group_totals")
             if totals is None or totals.device != idx.device:
-                totals = ws["group_totals"] = torch.empty(self.solver.n_experts, dtype=torch.int32, device=idx.device)
+                totals = ws["group_totals"] = torch.empty(n_experts, dtype=torch.int32, device=idx.device)
             workload = self.solver.count_totals(idx, out=totals)
         else:                                        # a long batch: histogram and scan
             table = ws.get("group_counts")
             if table is None or table.device != idx.device:
-                table = ws["group_counts"] = torch.empty((n_sms, self.solver.n_experts), dtype=torch.int32,
-                                                         device=idx.device)
+                table = ws["group_counts"] = torch.empty((n_sms, n_experts), dtype=torch.int32, device=idx.device)
             workload, _by_sm = self.solver.count_idx(idx, n_sms, 256, out=table)
         if not self.deep_ep_initialized:
             torch.distributed.all_reduce(workload, group=self.ep_group)

@@ -63,6 +63,36 @@ def _random_weights(shape: Shape, rng):
 
 
 @pytest.mark.parametrize("n,n_experts,offset", [(65536, 256, 0), (65537, 256, 1), (4099, 30, 0), (1, 7, 0), (0, 64, 0),
+                                                (131072, 256, 1), (100000, 2017, 0), (70000, 16384, 2), (8193, 5, 0)])
+def test_count_totals_add_swaps_two_vectors(cuda, n, n_experts, offset):
+    """lplb_count_totals_add: the batch's counts are added to a zeroed vector and the other vector comes back
+    zeroed, call after call with the two swapped; a second call into the same vector adds to what is there.
+    Masked and out-of-range values, odd lengths, views at an odd multiple of 8 bytes, one and eight LDS copies."""
+    rng = np.random.default_rng(n + n_experts)
+    solver = CompiledSolver(1, 1, 1, n_experts + 1, 1)
+    assert solver.n_experts == n_experts
+    pair = [torch.zeros(n_experts, dtype=torch.int32, device=cuda),
+            torch.full((n_experts,), 77, dtype=torch.int32, device=cuda)]       # (the other one starts dirty)
+    turn = 0
+    for call in range(3):
+        host = rng.integers(-1, n_experts, size=n + offset).astype(np.int64)
+        if n > 10:
+            host[offset + 3] = n_experts          # out of range: not counted
+            host[offset + 7] = -5
+            host[offset + 5:offset + 5 + n // 3] = (call * 7) % n_experts      # a hot expert
+        want = np.bincount(host[offset:][(host[offset:] >= 0) & (host[offset:] < n_experts)], minlength=n_experts)
+        got = solver.count_totals_add(dev(host, cuda)[offset:], pair[turn], clear=pair[1 - turn])
+        torch.cuda.synchronize()
+        assert got is pair[turn]
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+        assert int(pair[1 - turn].abs().max()) == 0
+        if call == 2:                             # once more into the same vector: the counts double
+            solver.count_totals_add(dev(host, cuda)[offset:], pair[turn])
+            np.testing.assert_array_equal(pair[turn].cpu().numpy(), 2 * want)
+        turn = 1 - turn
+
+
+@pytest.mark.parametrize("n,n_experts,offset", [(65536, 256, 0), (65537, 256, 1), (4099, 30, 0), (1, 7, 0), (0, 64, 0),
                                                 (131072, 1024, 3), (2, 3, 1), (50000, 257, 0)])
 def test_count_totals_matches_oracle(cuda, n, n_experts, offset):
     """The one-launch totals (what Planner.run feeds the all-reduce with) equal the last row of the table, for
@@ -1052,6 +1082,29 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
         assert int(avail[0]) == int(avail2[0]) == shape.n_group, (times, int(avail[0]), int(avail2[0]))
         assert torch.equal(got, want), (times, int((got != want).sum()))
     assert len(calls) == 4   # run, solve_probs, and the two runs above
+    # captured into a graph, the call must not rely on what an earlier call left in its vectors
+    # (LP and redirect as the chain of kernels here: a captured one-launch plan keeps its share of the GPU
+    # reserved for as long as the process lives, and this test is about the counts)
+    _native.set_plan_cooperative(False)
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            planner.run(t["idx"], avail, 256)                       # (buffers of this stream, outside the capture)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = planner.run(t["idx"], avail, 256)
+        for replay in range(3):
+            avail.zero_()
+            captured.fill_(-7)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(captured, out) and int(avail[0]) == shape.n_group, replay
+            planner.run(t["idx"], torch.zeros_like(avail), 256)     # eager work between the replays
+            torch.cuda.synchronize()
+    finally:
+        _native.set_plan_cooperative(True)
 
 
 @pytest.mark.parametrize("use_global", [True, False])

@@ -223,7 +223,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert sorted(_native.exported_symbols()) == declared
-    assert lib.lplb_abi_version() == _native.ABI_VERSION == 6
+    assert lib.lplb_abi_version() == _native.ABI_VERSION == 7
     header = (ROOT / "include" / "lplb_hip.h").read_text()
     assert f"#define LPLB_ABI_VERSION {_native.ABI_VERSION}" in header
     assert f"#define LPLB_COUNT_TOTALS_MAX_INDICES {_native.COUNT_TOTALS_MAX_INDICES}\n" in header
@@ -242,6 +242,12 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     assert lib.lplb_count_totals(p, 4, 0, p, None) == 1
     assert lib.lplb_count_totals(p, 4, 8, None, None) == 1
     assert lib.lplb_count_totals(p, 1 << 20, 8, p, None) == 2          # a long batch: histogram and scan serve it
+    assert lib.lplb_count_totals_add(p, 4, 0, p, None, None) == 1
+    assert lib.lplb_count_totals_add(p, 4, 8, None, None, None) == 1
+    assert lib.lplb_count_totals_add(p, 4, 8, p, p, None) == 1            # totals and clear are one vector
+    assert b"same vector" in lib.lplb_last_error()
+    assert lib.lplb_count_totals_add(p, 4, 1 << 20, p, None, None) == 2   # histogram does not fit LDS
+    assert lib.lplb_count_totals_add(p, 1 << 20, 8, p, None, None) == 2   # a long batch
     assert lib.lplb_solve(p, p, p, p, 1, 16, 9, 1, 2, p, p, 0, 5, None) == 2   # 144 edges > two per lane of a wave
     assert b"128 replica edges" in lib.lplb_last_error()
     assert lib.lplb_solve(p, p, p, p, 1, 4, 17, 1, 2, p, p, 0, 5, None) == 2   # more than 16 slots per rank
