@@ -663,10 +663,12 @@ def main() -> None:
         extras["planner_run_wall_us"] = wall_us_per_call(lambda: planner.run(idx, avail, n_sms))
         extras["planner_run_us_p50"] = round(pct(event_times_us(lambda: planner.run(idx, avail, n_sms), 1000, 100, torch), 50), 2)
 
-        # The same call on a Planner that was given a process group: histogram (lplb_count_idx), copy of the
-        # counts, all-reduce over the EP ranks, then LP and redirect as one plan on the summed counts.  One GPU:
-        # the all-reduce itself is left out (the stand-in group below is never handed to torch.distributed),
-        # everything around it runs as in a deployment.
+        # The same call on a Planner that was given a process group: this GPU's counts in one launch
+        # (lplb_count_totals_add), all-reduce over the EP ranks, then LP and redirect as one plan on the summed
+        # counts.  One GPU: the all-reduce itself is left out (the stand-in group below is never handed to
+        # torch.distributed), everything around it runs as in a deployment.  The call is two library calls and
+        # the host needs longer for them than the GPU: the wall figure is the sustained one, the event figure
+        # adds what recording an event between calls costs.
         class OneRankGroup:
             def size(self):
                 return cfg.ep_size
