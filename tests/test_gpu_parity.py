@@ -1056,12 +1056,18 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
         tensor += others.view_as(tensor)
 
     monkeypatch.setattr(torch.distributed, "all_reduce", fake_all_reduce)
+    took = []          # which of the three ways to this GPU's counts a call took
+    for way in ("count_totals_add", "count_totals", "count_idx"):
+        def spy(self, *a, _way=way, _real=getattr(CompiledSolver, way), **kw):
+            took.append(_way)
+            return _real(self, *a, **kw)
+        monkeypatch.setattr(CompiledSolver, way, spy)
     group = object()
     planner = Planner(torch.from_numpy(c.r2o), c.n_physical, c.n_logical, c.ep_size, group)
     planner.phy2log = t["phy2log"]
     avail = torch.zeros(1, dtype=torch.int32, device=cuda)
     out = planner.run(t["idx"], avail, 256)
-    assert calls == [group] and int(avail[0]) == shape.n_group
+    assert calls == [group] and int(avail[0]) == shape.n_group and took == ["count_totals_add"]
     summed = dev(local, cuda) + others
     avail2 = torch.zeros(1, dtype=torch.int32, device=cuda)
     want, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail2, 256, global_counts=summed)
@@ -1082,6 +1088,8 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
         assert int(avail[0]) == int(avail2[0]) == shape.n_group, (times, int(avail[0]), int(avail2[0]))
         assert torch.equal(got, want), (times, int((got != want).sum()))
     assert len(calls) == 4   # run, solve_probs, and the two runs above
+    assert took == ["count_totals_add", "count_idx", "count_idx", "count_totals_add"]   # (count_workload is the third)
+    took.clear()
     # captured into a graph, the call must not rely on what an earlier call left in its vectors
     # (LP and redirect as the chain of kernels here: a captured one-launch plan keeps its share of the GPU
     # reserved for as long as the process lives, and this test is about the counts)
@@ -1103,6 +1111,7 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
             assert torch.equal(captured, out) and int(avail[0]) == shape.n_group, replay
             planner.run(t["idx"], torch.zeros_like(avail), 256)     # eager work between the replays
             torch.cuda.synchronize()
+        assert took == ["count_totals_add", "count_totals"] + 3 * ["count_totals_add"]
     finally:
         _native.set_plan_cooperative(True)
 
