@@ -11,6 +11,8 @@
 // measured and rejected: one CU sustains too few outstanding misses to pull the
 // 256 KB table, 20 us against 3 us for this kernel.)
 // HBM-bound: 8 bytes read per index; the [n_blocks, n_experts] table is small.
+// Callers that need only the totals of a short batch get them in one launch: slice_histogram with
+// TOTALS (slices add their counts to one vector) or expert_totals (every workgroup owns four experts).
 #include "common.h"
 
 namespace lplb {
@@ -93,15 +95,15 @@ __global__ __launch_bounds__(1024) void slice_histogram(
     count(idx[end - 1]);
   __syncthreads();
   int32_t *row = TOTALS ? counts : counts + (int64_t)p * n_experts;
-  for (int e = tid; e < n_experts; e += nt) {
-    int32_t sum = 0;
+  if constexpr (!TOTALS) {
+    for (int e = tid; e < n_experts; e += nt) {
+      int32_t sum = 0;
 #pragma unroll
-    for (int k = 0; k < COPIES; ++k)
-      sum += hist[k * stride + e];
-    if constexpr (!TOTALS)
+      for (int k = 0; k < COPIES; ++k)
+        sum += hist[k * stride + e];
       row[e] = sum;
-  }
-  if constexpr (TOTALS) {
+    }
+  } else {
     // Two counters per atomic add: updates of one 64-byte line of memory are served one after the other
     // (about 14 ns each), and every slice updates every line, so the number of updates is what this
     // costs.  A counter stays below 2^31, so the low half never carries into the high one.
