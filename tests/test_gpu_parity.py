@@ -1117,6 +1117,21 @@ def test_planner_run_with_a_process_group(cuda, monkeypatch):
 
 
 @pytest.mark.parametrize("use_global", [True, False])
+def test_plan_at_the_sweep_shape_is_one_launch_and_equals_the_chain(cuda, use_global):
+    """[262144 x 8] indices: 256 slices of 8192 indices (16 chunks per wave) and the LP in one grid.
+    (Ahead of the tests that capture plans into graphs: a captured one-launch plan keeps its share of the GPU
+    reserved for as long as the process lives, and this plan needs a third of the GPU.)"""
+    inp = synth.make_inputs("sweep_redirect", mask_fraction=0.01)
+    got = _one_launch_equals_chain(cuda, inp, use_global, 512, expect_one_launch=True)
+    c = inp.cfg
+    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
+    by_sm = oracle.count_idx(inp.indices.reshape(-1), c.n_logical, 512)
+    want = oracle.map_idx(inp.indices.reshape(-1), got[1], by_sm, shape.o2r, inp.phy2log, shape.n_group, shape.C,
+                          shape.P).reshape(inp.indices.shape)
+    np.testing.assert_array_equal(got[0], want)
+
+
+@pytest.mark.parametrize("use_global", [True, False])
 @pytest.mark.parametrize("one_launch", [True, False])
 def test_plan_replays_from_a_hip_graph(cuda, use_global, one_launch):
     """Capture two plans into a graph; every replay, with eager work and synchronisation between
@@ -1257,19 +1272,6 @@ def test_one_launch_plan_while_another_stream_fills_the_gpu(cuda):
         del c
     assert _native.plan_sync_timeouts() == timeouts_before
     assert _native.plan_one_launch_count() - launches_before == 40     # not the chain by accident
-
-
-@pytest.mark.parametrize("use_global", [True, False])
-def test_plan_at_the_sweep_shape_is_one_launch_and_equals_the_chain(cuda, use_global):
-    """[262144 x 8] indices: 256 slices of 8192 indices (16 chunks per wave) and the LP in one grid."""
-    inp = synth.make_inputs("sweep_redirect", mask_fraction=0.01)
-    got = _one_launch_equals_chain(cuda, inp, use_global, 512, expect_one_launch=True)
-    c = inp.cfg
-    shape = Shape(c.r2o, c.ep_size, c.n_logical, c.n_physical)
-    by_sm = oracle.count_idx(inp.indices.reshape(-1), c.n_logical, 512)
-    want = oracle.map_idx(inp.indices.reshape(-1), got[1], by_sm, shape.o2r, inp.phy2log, shape.n_group, shape.C,
-                          shape.P).reshape(inp.indices.shape)
-    np.testing.assert_array_equal(got[0], want)
 
 
 @pytest.mark.parametrize("use_global", [True, False])
