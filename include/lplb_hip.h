@@ -375,6 +375,17 @@ int lplb_plan_noalloc(const int64_t *idx, int64_t n_elements,
 int lplb_plan_set_cooperative(int enabled);
 
 /*
+ * No counterpart in the reference.  A one-launch plan that was captured into a
+ * graph keeps its share of the GPU reserved, because a replay may come at any
+ * time (see lplb_plan).  A caller who has destroyed every graph that holds a plan
+ * captured on `stream` (on the current device), and whose replays have all ended,
+ * says so here: the share is given back and the stream's block of counters may
+ * pass to another stream.  Not needed where all graphs are captured on one
+ * stream (they share one reservation, the largest).
+ */
+int lplb_plan_forget_captured(lplb_stream_t stream);
+
+/*
  * No counterpart in the reference.  The workgroups of the one-launch plan wait
  * for each other with a bounded number of polls; *count receives how many waits
  * ran out on the current device since the library was loaded (0 in a healthy

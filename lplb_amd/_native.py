@@ -51,6 +51,7 @@ _SIGNATURES = {
     "lplb_prepare_mapping": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _i64, _vp]),
     "lplb_map_idx_prepared": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "lplb_plan_set_cooperative": (_i, [_i]),
+    "lplb_plan_forget_captured": (_i, [_vp]),
     "lplb_plan_sync_timeouts": (_i, [_vp]),
     "lplb_plan_poll_timeouts": (_i, [_vp, _vp]),
     "lplb_plan_one_launch_count": (_i, [_vp]),
@@ -97,6 +98,12 @@ def exported_symbols() -> list[str]:
 def set_plan_cooperative(enabled: bool) -> None:
     """Let ``plan`` run short batches as one kernel launch (default) or always as the chain of kernels."""
     _check(load().lplb_plan_set_cooperative(1 if enabled else 0))
+
+
+def plan_forget_captured(stream: "torch.cuda.Stream") -> None:
+    """Give back the share of the GPU that one-launch plans captured on ``stream`` keep reserved; for callers
+    who have destroyed every graph that holds such a plan."""
+    _check(load().lplb_plan_forget_captured(stream.cuda_stream))
 
 
 def plan_sync_timeouts() -> int:

@@ -995,6 +995,24 @@ extern "C" int lplb_plan_set_cooperative(int enabled) {
   return LPLB_OK;
 }
 
+extern "C" int lplb_plan_forget_captured(lplb_stream_t stream) {
+  using namespace lplb;
+  PlanDevice *d = nullptr;
+  const int rc = plan_device(&d);
+  if (rc != LPLB_OK)
+    return rc;
+  std::lock_guard<std::mutex> lock(g_plan_guard);
+  for (int i = 0; i < kSyncSlots; ++i) {
+    PlanSlot &ps = d->slots[i];
+    if (ps.used && ps.captured && ps.stream == static_cast<hipStream_t>(stream)) {
+      // back to a slot whose stream has nothing pending: it may serve this stream again or pass to another
+      ps.captured = ps.maybe_executing = false;
+      ps.cost = 0.0f;
+    }
+  }
+  return LPLB_OK;
+}
+
 extern "C" int lplb_plan_sync_timeouts(int *count) {
   using namespace lplb;
   LPLB_REQUIRE(count != nullptr, LPLB_EINVAL, "plan_sync_timeouts: null pointer");

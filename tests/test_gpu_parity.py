@@ -1217,6 +1217,41 @@ def test_planner_run_replays_from_a_hip_graph(cuda):
         assert int(avail[0]) == before + 2 * (rep + 1)
 
 
+def test_forgetting_captured_plans_gives_their_share_back(cuda):
+    """Plans captured on stream after stream fill the library's eight blocks of counters, and later plans on a new
+    stream run as the chain; once the graphs are gone and the caller has said so, they run as one launch again."""
+    from lplb_amd import _native
+    inp, shape, solver, t = _plan_setup(cuda, "v3_ep8_cube")
+    avail = torch.zeros(1, dtype=torch.int32, device=cuda)
+
+    def plan_on(stream):
+        before = _native.plan_one_launch_count()
+        with torch.cuda.stream(stream):
+            out, _, _ = solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])
+        stream.synchronize()
+        return out, _native.plan_one_launch_count() - before
+
+    torch.cuda.synchronize()
+    want, one = plan_on(torch.cuda.Stream())
+    assert one == 1
+    streams, graphs = [], []
+    for _ in range(10):                          # more than there are blocks
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        plan_on(s)                               # (buffers and first-call work outside the capture)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            solver.plan(t["idx"], t["r2o"], t["o2r"], t["phy2log"], avail, 256, global_counts=t["counts"])
+        streams.append(s), graphs.append(g)
+    out, one = plan_on(torch.cuda.Stream())
+    assert one == 0 and torch.equal(out, want)   # no block left, or no room beside the reserved shares: the chain
+    del graphs
+    for s in streams:
+        _native.plan_forget_captured(s)
+    out, one = plan_on(torch.cuda.Stream())
+    assert one == 1 and torch.equal(out, want)
+
+
 @pytest.mark.parametrize("cooperative", [False, True])
 def test_plans_on_two_streams(cuda, cooperative):
     """Plans on different streams may overlap on the device.  The one-launch form keeps its
