@@ -304,7 +304,7 @@ int lplb_map_idx_prepared(const int64_t *idx, const float *o_weight,
  * those words: it never waits and never hands a stream of the caller's to the runtime
  * after the call that brought it); otherwise the call runs the
  * chain, with identical results.  A plan captured into a graph keeps its share of the GPU reserved
- * from then on (its replays are invisible to the library).  Launches on one stream never overlap; the exception the
+ * from then on (its replays are invisible to the library; see lplb_plan_forget_captured).  Launches on one stream never overlap; the exception the
  * library cannot see is a graph captured on one stream and replayed concurrently on
  * several (see lplb_plan_set_cooperative).  Every wait inside the kernel is bounded; if one
  * runs out, the launch still completes, with a valid but unbalanced result: the tokens of
